@@ -203,6 +203,118 @@ NV_API int nv_moe_down(const void* y, const void* down, const int32_t* sorted_pa
                        const float* pair_weights, float* out, int dtype, int64_t pairs, int E, int width, int ff,
                        int tile_rows, void* stream);
 
+/* nv_causal_conv_silu with a bias [C] (fp32, may be NULL) added to the convolution before the SiLU. */
+NV_API int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const float* w, const float* bias, void* conv_state,
+                                    void* y, int64_t y_stride, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                    const int32_t* state_slots, int num_seqs, int64_t T, int C, int taps, int dtype,
+                                    void* stream);
+
+/* nv_moe_gate_up with a free shift of the up branch: act = g * sigmoid(alpha g) * (u + up_shift); limit = +inf, alpha = 1,
+ * up_shift = 0 is the plain SiLU-gated unit. */
+NV_API int nv_moe_gate_up_act(const void* h, int64_t h_stride, const void* gate_up, const int32_t* sorted_pairs,
+                              const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width, int ff,
+                              float limit, float alpha, float up_shift, int tile_rows, void* stream);
+
+/*
+ * Embedding with a hashed bigram table, RMS-normed into an fp32 stream x [T, cols]:
+ *   x[t] = rmsnorm(embed[id_t] + bigram[row_t]) * norm_w,  row_t = (id_{t-1} * mul_prev + id_t * mul_cur) mod buckets,
+ *   or row `buckets` at position 0.  prev_state [num_slots] int64 carries each sequence's last id between steps.
+ *   bigram NULL: the embedding row alone.  embed: [vocab, cols], bigram: [buckets + 1, cols] of dtype.
+ */
+NV_API int nv_hashed_bigram_embed(const int64_t* ids, const int64_t* positions, const void* embed, const void* bigram,
+                                  int64_t buckets, int64_t mul_prev, int64_t mul_cur, const float* norm_w, float eps,
+                                  int64_t* prev_state, float* x, const int32_t* cu_seqlens_q, const int32_t* state_slots,
+                                  int num_seqs, int64_t T, int cols, int dtype, void* stream);
+
+/*
+ * One layer boundary of an fp32 stream that is read through two RMS norms, per row and in place:
+ *   r += add1 + add2 + parts_scale * sum_j parts[:, j]                          (each may be NULL / absent)
+ *   r += normed_mult * (rmsnorm(normed1) * normed1_w + rmsnorm(normed2) * normed2_w)      (each may be NULL)
+ *   y32[:, :cols] = rmsnorm(r) * norm_a;  y32[:, cols:] = rmsnorm(r) * norm_b    (norm_b NULL: y32 is [rows, cols])
+ *   y = rmsnorm(r) * norm_a in dtype                                             (y32 and / or y)
+ * add*, normed*: [rows, cols] of dtype with row strides; parts: [rows, n_parts, cols] fp32.
+ */
+NV_API int nv_stream_boundary_pair(void* resid, const void* add1, int64_t add1_stride, const void* add2,
+                                   int64_t add2_stride, const float* parts, int n_parts, float parts_scale,
+                                   const void* normed1, int64_t normed1_stride, const float* normed1_w,
+                                   const void* normed2, int64_t normed2_stride, const float* normed2_w, float normed_mult,
+                                   const float* norm_a, const float* norm_b, float eps, float* y32, void* y, int dtype,
+                                   int64_t rows, int cols, void* stream);
+
+/* y = max(x, 0)^2; x: [rows, cols] with a row stride, y contiguous. */
+NV_API int nv_relu_squared(const void* x, int64_t x_stride, void* y, int dtype, int64_t rows, int cols, void* stream);
+
+/*
+ * Decayed outer-product memory read BEFORE it is written, with a bonus for the current token; state
+ * [num_slots, H, Dk, Dv] fp32 carried per slot:
+ *   w = exp(-exp(w_raw + w_bias));  o = (S + diag(bonus) k v^T)^T r;  S <- diag(w) S + k v^T      (token by token)
+ *   out[t, h] = o / sqrt(mean(o^2) + eps) * norm_w[h] * silu(gate_raw[t, h])
+ * r, k, w_raw: [T, H, Dk]; v, gate_raw, out: [T, H, Dv] of dtype with token strides; w_bias, bonus: [H, Dk] fp32;
+ * norm_w: [H, Dv] fp32.  Dk, Dv <= 256.
+ */
+NV_API int nv_decay_memory(const void* r, const void* k, const void* v, int64_t r_stride, int64_t k_stride,
+                           int64_t v_stride, const void* w_raw, int64_t w_stride, const void* gate_raw,
+                           int64_t gate_stride, const float* w_bias, const float* bonus, const float* norm_w, float* state,
+                           void* out, int64_t out_stride, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                           const int32_t* state_slots, int num_seqs, int H, int Dk, int Dv, float eps, int dtype,
+                           void* stream);
+
+/*
+ * State-space scan with one scalar decay per head and step; state [num_slots, H, N, P] fp32 carried per slot:
+ *   dt = softplus(dt_raw + dt_bias);  S <- exp(-exp(A_log) dt) S + dt B x^T;  y = S^T C + D x;  out = y * silu(z)
+ * x, z: [T, H, P]; B, C: [T, G, N] (head h reads group h / (H / G)); dt_raw: [T, H] of dtype with token strides;
+ * dt_bias, A_log, D: [H] fp32; out: [T, H * P] fp32 (a grouped norm follows).  N, P <= 256.
+ */
+NV_API int nv_state_space_scan(const void* x, const void* B, const void* C, int64_t x_stride, int64_t b_stride,
+                               int64_t c_stride, const void* dt_raw, int64_t dt_stride, const void* z, int64_t z_stride,
+                               const float* dt_bias, const float* A_log, const float* D_skip, float* state, float* out,
+                               int64_t out_stride, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                               const int32_t* state_slots, int num_seqs, int H, int G, int N, int P, int dtype,
+                               void* stream);
+
+/*
+ * out[s, t] = h[t] + (h[t-1] - h[t]) * mu[s] for n_mix blends at once; the row before a sequence's first row of the
+ * step comes from state[slot] (zeros at position 0), which then takes the step's last row.  h: [T, C] of dtype with a
+ * row stride; mu: [n_mix, C] fp32; state: [num_slots, C] of dtype; out: [n_mix, T, C] of dtype.
+ */
+NV_API int nv_token_shift_mix(const void* h, int64_t h_stride, const float* mu, int n_mix, void* state, void* out,
+                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* state_slots,
+                              int num_seqs, int64_t T, int C, int dtype, void* stream);
+
+/* y = x / sqrt(mean(part^2) + eps) * w over `groups` equal consecutive parts of every fp32 row; y of y_dtype. */
+NV_API int nv_group_rms_norm(const float* x, int64_t x_stride, const float* w, void* y, int64_t y_stride, int y_dtype,
+                             int64_t rows, int cols, int groups, float eps, void* stream);
+
+/*
+ * In front of nv_attn_chunk_sigmoid_paged: RMS norm over the whole q row [H * D] and the whole k row [G * D] (weights
+ * q_norm, k_norm of those sizes), rotate-half rotary on the first rot_dims dimensions of every head (pair (i, i +
+ * rot_dims / 2) by positions[t] * freq[i]), every value head turned the same way over all Dv dimensions by positions[t] *
+ * value_freq[m], and the scatter of the rotated k / v rows into the paged caches.  q_out: [T, H, D] contiguous.
+ */
+NV_API int nv_chunk_attn_prep_store(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                                    int64_t v_stride, const float* q_norm, const float* k_norm, float eps,
+                                    const float* freq, int rot_dims, const float* value_freq, const int64_t* positions,
+                                    const int32_t* slot_mapping, void* q_out, void* k_cache, void* v_cache, int dtype,
+                                    int64_t T, int H, int G, int D, int Dv, void* stream);
+
+/*
+ * Sigmoid attention inside chunks of `chunk` positions (0: plain causal) over a paged cache of ROTATED values:
+ *   out[i] = R(-i) sum_{j <= i, same chunk} sigmoid(scale q_i . k_j + head_bias[h]) v_cache[j]
+ * R(p) turns the pair (m, m + Dv / 2) by p * value_freq[m].  q: [T, H, D]; caches [num_blocks, block_size, G, D | Dv];
+ * out: [T, H * Dv].  tile_seq / tile_q0 [num_tiles] (may be 0 tiles): blocks of 64 query rows of sequences with several
+ * rows, for the bf16 MFMA kernel (nv_attn_chunk_sigmoid_tile_ok says whether it is built for the sizes); with tiles,
+ * single_rows != 0 says that the step also has sequences with one row.  Without tiles every row takes the
+ * one-wave-per-row kernel.
+ */
+NV_API int nv_attn_chunk_sigmoid_tile_ok(int D, int Dv, int dtype);
+NV_API int nv_attn_chunk_sigmoid_paged(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                       const int32_t* block_tables, int num_seqs, int max_blocks, int64_t T, int H, int G,
+                                       int D, int Dv, int64_t num_blocks, int block_size, float scale,
+                                       const float* head_bias, int chunk, const float* value_freq,
+                                       const int32_t* tile_seq, const int32_t* tile_q0, int num_tiles, int single_rows,
+                                       int dtype, int64_t q_stride, int64_t out_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip.so")
 MIXERS_LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip_mixers.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -95,6 +95,27 @@ MIXERS_PROTOTYPES = {
     "nv_moe_align": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "nv_moe_gate_up": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _i32, _vp]),
     "nv_moe_down": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "nv_moe_gate_up_act": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _i32,
+                                  _vp]),
+    "nv_causal_conv_bias_silu": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32,
+                                        _vp]),
+    "nv_hashed_bigram_embed": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _i32, _i64, _i32,
+                                      _i32, _vp]),
+    "nv_stream_boundary_pair": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i32, _f32, _vp, _i64, _vp, _vp, _i64, _vp, _f32, _vp,
+                                       _vp, _f32, _vp, _vp, _i32, _i64, _i32, _vp]),
+    "nv_relu_squared": (_i32, [_vp, _i64, _vp, _i32, _i64, _i32, _vp]),
+    "nv_decay_memory": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp,
+                               _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "nv_state_space_scan": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64,
+                                   _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "nv_token_shift_mix": (_i32, [_vp, _i64, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp]),
+    "nv_group_rms_norm": (_i32, [_vp, _i64, _vp, _vp, _i64, _i32, _i64, _i32, _i32, _f32, _vp]),
+    "nv_chunk_attn_prep_store": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _f32, _vp, _i32, _vp, _vp, _vp, _vp,
+                                        _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "nv_attn_chunk_sigmoid_tile_ok": (_i32, [_i32, _i32, _i32]),
+    "nv_attn_chunk_sigmoid_paged": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i32, _i32,
+                                           _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _i64,
+                                           _vp]),
 }
 DTYPE_BF16, DTYPE_F32 = 0, 1
 

@@ -37,9 +37,9 @@ __device__ __forceinline__ float softplus_f(float x) { return x > 20.0f ? x : lo
 
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
-    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const T* __restrict__ conv_state,
-    T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
-    const int* __restrict__ state_slots, int B, int C, int taps) {
+    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const float* __restrict__ bias,
+    const T* __restrict__ conv_state, T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q,
+    const int* __restrict__ cu_k, const int* __restrict__ state_slots, int B, int C, int taps) {
     const int t = blockIdx.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= C) return;
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     const int i = t - cu_q[b];
     const int start = (cu_k[b + 1] - cu_k[b]) - (cu_q[b + 1] - cu_q[b]);
     const T* st = conv_state + (int64_t)state_slots[b] * (taps - 1) * C;
-    float acc = 0.f;
+    float acc = bias != nullptr ? bias[c] : 0.f;
     for (int j = 0; j < taps; ++j) {
         const int src = i - j;
         float xv = 0.f;
@@ -91,13 +91,17 @@ template <> struct Piece<float> {
 // the carried state (or zeros before position 0).
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_silu_pieces_kernel(
-    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const T* __restrict__ conv_state,
-    T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
-    const int* __restrict__ state_slots, int B, int C, int taps, int T_rows, int tokens_per_group) {
+    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const float* __restrict__ bias,
+    const T* __restrict__ conv_state, T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q,
+    const int* __restrict__ cu_k, const int* __restrict__ state_slots, int B, int C, int taps, int T_rows,
+    int tokens_per_group) {
     constexpr int N = Piece<T>::n;
     const int c = (blockIdx.y * 256 + threadIdx.x) * N;
     if (c >= C) return;
     float wt[kConvMaxTaps][N], win[kConvMaxTaps][N];        // wt[j], win[j]: weight of / input at the token j back
+    float bs[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) bs[e] = bias != nullptr ? bias[c + e] : 0.f;
 #pragma unroll
     for (int j = 0; j < kConvMaxTaps; ++j) {
 #pragma unroll
@@ -138,7 +142,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_pieces_kernel(
         Piece<T>::load(x + (int64_t)t * x_stride + c, win[0]);
         float acc[N];
 #pragma unroll
-        for (int e = 0; e < N; ++e) acc[e] = 0.f;
+        for (int e = 0; e < N; ++e) acc[e] = bs[e];
 #pragma unroll
         for (int j = 0; j < kConvMaxTaps; ++j) {
 #pragma unroll
@@ -352,6 +356,14 @@ extern "C" int nv_causal_conv_silu(const void* x, int64_t x_stride, const float*
                                    int64_t y_stride, const int* cu_seqlens_q, const int* cu_seqlens_k,
                                    const int* state_slots, int num_seqs, int64_t T, int C, int taps, int dtype,
                                    void* stream) {
+    return nv_causal_conv_bias_silu(x, x_stride, w, nullptr, conv_state, y, y_stride, cu_seqlens_q, cu_seqlens_k,
+                                    state_slots, num_seqs, T, C, taps, dtype, stream);
+}
+
+extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const float* w, const float* bias,
+                                        void* conv_state, void* y, int64_t y_stride, const int* cu_seqlens_q,
+                                        const int* cu_seqlens_k, const int* state_slots, int num_seqs, int64_t T, int C,
+                                        int taps, int dtype, void* stream) {
     using namespace nv;
     NV_REQUIRE(num_seqs >= 0 && T >= 0 && C > 0, NV_ERR_INVALID_ARG, "nv_causal_conv_silu: bad sizes");
     NV_REQUIRE(taps >= 1 && taps <= kConvMaxTaps, NV_ERR_UNSUPPORTED, "nv_causal_conv_silu: taps=%d not in 1..%d", taps,
@@ -371,11 +383,11 @@ extern "C" int nv_causal_conv_silu(const void* x, int64_t x_stride, const float*
     if (dtype == NV_DTYPE_BF16) {
         if (pieces)
             hipLaunchKernelGGL(causal_conv_silu_pieces_kernel<__bf16>, dim3((unsigned)((T + tpg - 1) / tpg), pb), dim3(256), 0, s,
-                               (const __bf16*)x, x_stride, w, (const __bf16*)conv_state, (__bf16*)y, y_stride,
+                               (const __bf16*)x, x_stride, w, bias, (const __bf16*)conv_state, (__bf16*)y, y_stride,
                                cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg);
         else
         hipLaunchKernelGGL(causal_conv_silu_kernel<__bf16>, dim3((unsigned)T, cb), dim3(256), 0, s, (const __bf16*)x,
-                           x_stride, w, (const __bf16*)conv_state, (__bf16*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
+                           x_stride, w, bias, (const __bf16*)conv_state, (__bf16*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
                            state_slots, num_seqs, C, taps);
         if (taps > 1)
             hipLaunchKernelGGL(conv_state_update_kernel<__bf16>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
@@ -384,11 +396,11 @@ extern "C" int nv_causal_conv_silu(const void* x, int64_t x_stride, const float*
     } else {
         if (pieces)
             hipLaunchKernelGGL(causal_conv_silu_pieces_kernel<float>, dim3((unsigned)((T + tpg - 1) / tpg), pb), dim3(256), 0, s,
-                               (const float*)x, x_stride, w, (const float*)conv_state, (float*)y, y_stride,
+                               (const float*)x, x_stride, w, bias, (const float*)conv_state, (float*)y, y_stride,
                                cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg);
         else
         hipLaunchKernelGGL(causal_conv_silu_kernel<float>, dim3((unsigned)T, cb), dim3(256), 0, s, (const float*)x,
-                           x_stride, w, (const float*)conv_state, (float*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
+                           x_stride, w, bias, (const float*)conv_state, (float*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
                            state_slots, num_seqs, C, taps);
         if (taps > 1)
             hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,

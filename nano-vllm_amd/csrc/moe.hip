@@ -148,7 +148,7 @@ template <typename T, int MT, int NT, bool GATE_UP>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, const int* __restrict__ sorted_pairs,
     const int* __restrict__ meta, const float* __restrict__ pair_w, T* __restrict__ y, float* __restrict__ out, int top,
-    int N, int K, float limit, float alpha, int vec_ok, int max_tiles) {
+    int N, int K, float limit, float alpha, float up_shift, int vec_ok, int max_tiles) {
     using M = MoeMma<T>;
     constexpr int BK = M::kBK, BM = 16 * MT, BN = 64 * NT, NB = GATE_UP ? 2 : 1, LD = BK + M::kPad, KV = BK / M::kVec;
     constexpr int A_IT = (BM * KV + 255) / 256, B_IT = (NB * BN * KV + 255) / 256;
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
                 if constexpr (GATE_UP) {
                     const float g = fminf(acc[nt][m][i], limit);
                     const float u = fminf(fmaxf(acc[NT + nt][m][i], -limit), limit);
-                    y[(int64_t)(row0 + r) * N + n] = (T)(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+                    y[(int64_t)(row0 + r) * N + n] = (T)(g / (1.0f + expf(-alpha * g)) * (u + up_shift));
                 } else {
                     const int pair = src_row[r];
                     out[(int64_t)pair * N + n] = acc[nt][m][i] * pair_w[pair];
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 template <typename T, bool GATE_UP>
 static void launch_grouped(const void* a, int64_t a_stride, const void* w, const int* sorted_pairs, const int* meta,
                            const float* pair_w, void* y, float* out, int top, int N, int K, float limit, float alpha,
-                           int max_tiles, int tile_rows, hipStream_t s) {
+                           float up_shift, int max_tiles, int tile_rows, hipStream_t s) {
     const int vec = MoeMma<T>::kVec;
     const int vec_ok = K % vec == 0 && a_stride % vec == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0;
     // many rows per expert: 64 x 128 tiles (a wave owns 32 columns; 128-row tiles measured slower: one workgroup per CU);
@@ -256,7 +256,7 @@ static void launch_grouped(const void* a, int64_t a_stride, const void* w, const
 #define NV_MOE_LAUNCH(MT, NT)                                                                                          \
     hipLaunchKernelGGL((moe_grouped_kernel<T, MT, NT, GATE_UP>), dim3((unsigned)(max_tiles * ((N + 64 * NT - 1) / (64 * NT)))), \
                        dim3(256), 0, s, (const T*)a, a_stride, (const T*)w, sorted_pairs, meta, pair_w, (T*)y, out, top, N, K,  \
-                       limit, alpha, vec_ok, max_tiles)
+                       limit, alpha, up_shift, vec_ok, max_tiles)
     if (tile_rows == 64 && sizeof(T) == 2) NV_MOE_LAUNCH(4, 2);
     else if (tile_rows == 64) NV_MOE_LAUNCH(4, 1);
     else NV_MOE_LAUNCH(1, 1);
@@ -298,6 +298,13 @@ extern "C" int nv_moe_align(const int32_t* ids, int32_t* sorted_pairs, int32_t* 
 extern "C" int nv_moe_gate_up(const void* h, int64_t h_stride, const void* gate_up, const int32_t* sorted_pairs,
                               const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width, int ff,
                               float limit, float alpha, int tile_rows, void* stream) {
+    return nv_moe_gate_up_act(h, h_stride, gate_up, sorted_pairs, meta, y, dtype, pairs, E, top, width, ff, limit, alpha,
+                              1.0f, tile_rows, stream);
+}
+
+extern "C" int nv_moe_gate_up_act(const void* h, int64_t h_stride, const void* gate_up, const int32_t* sorted_pairs,
+                                  const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width,
+                                  int ff, float limit, float alpha, float up_shift, int tile_rows, void* stream) {
     using namespace nv;
     NV_REQUIRE(pairs >= 0 && E > 0 && top > 0 && width > 0 && ff > 0 && (tile_rows == 16 || tile_rows == 64),
                NV_ERR_INVALID_ARG, "nv_moe_gate_up: bad sizes");
@@ -309,10 +316,10 @@ extern "C" int nv_moe_gate_up(const void* h, int64_t h_stride, const void* gate_
     hipStream_t s = (hipStream_t)stream;
     if (dtype == NV_DTYPE_BF16)
         launch_grouped<__bf16, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
-                                     alpha, (int)tiles, tile_rows, s);
+                                     alpha, up_shift, (int)tiles, tile_rows, s);
     else
         launch_grouped<float, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
-                                    alpha, (int)tiles, tile_rows, s);
+                                    alpha, up_shift, (int)tiles, tile_rows, s);
     return check_launch("nv_moe_gate_up");
 }
 
@@ -329,10 +336,10 @@ extern "C" int nv_moe_down(const void* y, const void* down, const int32_t* sorte
     NV_REQUIRE(tiles * ((width + kMoeBN - 1) / kMoeBN) < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_down: launch too large");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == NV_DTYPE_BF16)
-        launch_grouped<__bf16, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f,
+        launch_grouped<__bf16, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f, 0.f,
                                       (int)tiles, tile_rows, s);
     else
-        launch_grouped<float, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f,
+        launch_grouped<float, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f, 0.f,
                                      (int)tiles, tile_rows, s);
     return check_launch("nv_moe_down");
 }

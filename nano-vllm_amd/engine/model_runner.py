@@ -316,7 +316,8 @@ class ModelRunner:
                            num_leading_decode=m["num_leading_decode"], max_seqlen_k_decode=m["max_seqlen_k_decode"],
                            max_seqlen_q_rest=m["max_seqlen_q_rest"], max_seqlen_k_rest=m["max_seqlen_k_rest"],
                            decode_chunk_keys=self._decode_chunk(m, m["max_seqlen_k_decode"]),
-                           state_slots=self._to_device(m["state_slots"]) if self.has_state else None)
+                           state_slots=self._to_device(m["state_slots"]) if self.has_state else None,
+                           cu_seqlens_q_host=m["cu_seqlens_q"])
         set_context(ctx)
         return self._to_device(m["input_ids"]), self._to_device(m["positions"]), m
 

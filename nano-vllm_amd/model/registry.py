@@ -99,8 +99,19 @@ def _benarax_model(cfg, dtype=torch.bfloat16, device="cuda", **kw):
     return BenaraxForCausalLM(cfg, dtype=dtype, device=device, **kw)
 
 
+def _divadra_config(raw: dict):
+    from .divadra import DivadraConfig
+    return DivadraConfig.from_dict(raw)
+
+
+def _divadra_model(cfg, dtype=torch.bfloat16, device="cuda", **kw):
+    from .divadra import DivadraForCausalLM
+    return DivadraForCausalLM(cfg, dtype=dtype, device=device, **kw)
+
+
 register(["Qwen3ForCausalLM", "Qwen3"], _qwen3_config, lambda cfg, **kw: _qwen3_model(cfg, **kw))
 register(["LlamaForCausalLM", "Llama"], lambda raw: _qwen3_config({**raw, "qk_norm": False}),
          lambda cfg, **kw: _qwen3_model(cfg, **kw))
 register(["Buvalix", "BuvalixForCausalLM"], _buvalix_config, _buvalix_model)
 register(["Benarax", "BenaraxForCausalLM"], _benarax_config, _benarax_model)
+register(["Divadra", "DivadraForCausalLM"], _divadra_config, _divadra_model)

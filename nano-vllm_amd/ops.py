@@ -786,3 +786,346 @@ def moe_experts(h: torch.Tensor, logits: torch.Tensor, gate_up: torch.Tensor, do
     _lib.check(dll.nv_moe_down(y.data_ptr(), down.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), wgt.data_ptr(),
                                out.data_ptr(), dt, P, E, W, ff, rows, s), "nv_moe_down", dll)
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------
+# fp32 stream read through two RMS norms, hashed bigram embedding, decayed outer-product memories (bonus form and
+# state-space scan), token-shift blends, chunked sigmoid attention with rotated values, table-routed experts.
+# ---------------------------------------------------------------------------------------------------------
+def _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots):
+    for t, n in ((cu_seqlens_q, "cu_seqlens_q"), (cu_seqlens_k, "cu_seqlens_k"), (state_slots, "state_slots")):
+        _i32(t, n)
+    B = state_slots.numel()
+    _need(cu_seqlens_q.numel() == B + 1 and cu_seqlens_k.numel() == B + 1, "one state slot per sequence")
+    return B
+
+
+def hashed_bigram_embed(ids: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, bigram: Optional[torch.Tensor],
+                        mul_prev: int, mul_cur: int, norm_weight: torch.Tensor, eps: float,
+                        prev_state: Optional[torch.Tensor], cu_seqlens_q: torch.Tensor,
+                        state_slots: Optional[torch.Tensor]) -> torch.Tensor:
+    """x = rmsnorm(embed[id] + bigram[hash(previous id, id)]) * norm_weight as a float32 stream [T, W]; the last row
+    of the bigram table serves position 0; prev_state [slots] int64 carries each sequence's last id."""
+    dt = _dt(embed, "embed")
+    T, W = ids.numel(), embed.shape[1]
+    for t, n in ((ids, "ids"), (positions, "positions")):
+        _need(t.is_cuda and t.dtype == torch.int64 and t.is_contiguous() and t.numel() == T,
+              f"{n} must be a contiguous int64 [tokens] GPU tensor")
+    _need(embed.is_contiguous() and embed.dim() == 2, "embed must be contiguous [vocab, width]")
+    _i32(cu_seqlens_q, "cu_seqlens_q")
+    B = cu_seqlens_q.numel() - 1
+    buckets = 0
+    if bigram is not None:
+        _need(bigram.is_cuda and bigram.is_contiguous() and bigram.dtype == embed.dtype and bigram.shape[1] == W
+              and bigram.shape[0] >= 2, "bigram must be contiguous [buckets + 1, width] of embed's dtype")
+        buckets = bigram.shape[0] - 1
+        _need(prev_state is not None and prev_state.is_cuda and prev_state.dtype == torch.int64 and prev_state.is_contiguous(),
+              "prev_state must be a contiguous int64 [slots] GPU tensor")
+        _i32(state_slots, "state_slots")
+        _need(state_slots.numel() == B, "one state slot per sequence")
+    x = torch.empty((T, W), dtype=torch.float32, device=embed.device)
+    dll = _lib.mixers()
+    rc = dll.nv_hashed_bigram_embed(ids.data_ptr(), positions.data_ptr(), embed.data_ptr(), _ptr(bigram), buckets,
+                                    int(mul_prev), int(mul_cur), _f32c(norm_weight, "norm_weight"), float(eps),
+                                    _ptr(prev_state) if bigram is not None else None, x.data_ptr(),
+                                    cu_seqlens_q.data_ptr(), _ptr(state_slots) if bigram is not None else None, B, T, W,
+                                    dt, _stream(embed))
+    _lib.check(rc, "nv_hashed_bigram_embed", dll)
+    return x
+
+
+def stream_boundary_pair(x: torch.Tensor, adds=(), parts: Optional[torch.Tensor] = None, parts_scale: float = 1.0,
+                         normed=(), normed_mult: float = 1.0, norms=(), eps: float = 1e-5,
+                         out_dtype: Optional[torch.dtype] = None, want_f32: bool = True):
+    """One layer boundary of an fp32 stream x [T, W], in place:
+    x += sum(adds) + parts_scale * parts.sum(1) + normed_mult * sum(rmsnorm(n) * w for (n, w) in normed).
+    norms: up to two RMS-norm weights of the updated stream.  Returns (h32, h): the norms side by side in float32
+    [T, len(norms) * W] (if want_f32) and the FIRST norm in out_dtype (if given); None for each part not asked for."""
+    _need(x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(),
+          "the stream must be a contiguous float32 [tokens, width] GPU tensor")
+    rows, cols = x.shape
+    adds, normed, norms = list(adds), list(normed), list(norms)
+    _need(len(adds) <= 2 and len(normed) <= 2 and len(norms) <= 2, "at most two of each kind")
+    ins = adds + [n for n, _ in normed]
+    dt_t = out_dtype or (ins[0].dtype if ins else torch.float32)
+    _need(dt_t in (_BF16, torch.float32), "the matmul dtype must be bfloat16 or float32")
+    dt = _lib.DTYPE_BF16 if dt_t == _BF16 else _lib.DTYPE_F32
+    for t in ins:
+        _rows2d(t, "input")
+        _need(t.shape == x.shape and t.dtype == dt_t and t.is_cuda, "inputs must match the stream's shape, in the matmul dtype")
+    n_parts = 0
+    if parts is not None:
+        _need(parts.is_cuda and parts.dtype == torch.float32 and parts.is_contiguous() and parts.dim() == 3
+              and parts.shape[0] == rows and parts.shape[2] == cols, "parts must be contiguous float32 [T, n, W]")
+        n_parts = parts.shape[1]
+    for _, w in normed:
+        _need(w.numel() == cols, "a normed input needs its [width] weight")
+    for w in norms:
+        _need(w.numel() == cols, "norm weights must be [width]")
+    y32 = y = None
+    if norms:
+        if want_f32:
+            y32 = torch.empty((rows, len(norms) * cols), dtype=torch.float32, device=x.device)
+        if out_dtype is not None:
+            y = torch.empty((rows, cols), dtype=out_dtype, device=x.device)
+        _need(y32 is not None or y is not None, "the norm needs an output")
+    a1 = adds[0] if len(adds) > 0 else None
+    a2 = adds[1] if len(adds) > 1 else None
+    n1, w1 = normed[0] if len(normed) > 0 else (None, None)
+    n2, w2 = normed[1] if len(normed) > 1 else (None, None)
+    dll = _lib.mixers()
+    rc = dll.nv_stream_boundary_pair(x.data_ptr(), _ptr(a1), a1.stride(0) if a1 is not None else 0, _ptr(a2),
+                                     a2.stride(0) if a2 is not None else 0, _ptr(parts) if n_parts else None, n_parts,
+                                     float(parts_scale), _ptr(n1), n1.stride(0) if n1 is not None else 0,
+                                     _f32c(w1, "normed weight") or None, _ptr(n2), n2.stride(0) if n2 is not None else 0,
+                                     _f32c(w2, "normed weight") or None, float(normed_mult),
+                                     _f32c(norms[0], "norm") if norms else None,
+                                     _f32c(norms[1], "norm") if len(norms) > 1 else None, float(eps), _ptr(y32), _ptr(y),
+                                     dt, rows, cols, _stream(x))
+    _lib.check(rc, "nv_stream_boundary_pair", dll)
+    return y32, y
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    """max(x, 0)^2, x [T, C] bfloat16 or float32 (fp32 arithmetic, one rounding)."""
+    dt = _dt(x, "x")
+    _rows2d(x, "x")
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    _lib.check(dll.nv_relu_squared(x.data_ptr(), x.stride(0), y.data_ptr(), dt, x.shape[0], x.shape[1], _stream(x)),
+               "nv_relu_squared", dll)
+    return y
+
+
+def causal_conv_bias_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], conv_state: torch.Tensor,
+                          cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor) -> torch.Tensor:
+    """silu(causal conv over time + bias) per channel of x [T, C]; weight [C, taps] and bias [C] float32; conv_state
+    [num_slots, taps - 1, C] (x's dtype) carries each sequence's last inputs and is updated."""
+    dt = _dt(x, "x")
+    _rows2d(x, "x")
+    T, Cc = x.shape
+    taps = weight.shape[1]
+    _need(weight.shape[0] == Cc and (bias is None or bias.numel() == Cc), "weight must be [channels, taps], bias [channels]")
+    _need(conv_state.is_cuda and conv_state.dtype == x.dtype and conv_state.is_contiguous()
+          and conv_state.shape[1:] == (taps - 1, Cc), "conv_state must be contiguous [slots, taps - 1, C] of x's dtype")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    y = torch.empty((T, Cc), dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_causal_conv_bias_silu(x.data_ptr(), x.stride(0), _f32c(weight, "weight"), _f32c(bias, "bias") or None,
+                                      conv_state.data_ptr(), y.data_ptr(), y.stride(0), cu_seqlens_q.data_ptr(),
+                                      cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, T, Cc, taps, dt, _stream(x))
+    _lib.check(rc, "nv_causal_conv_bias_silu", dll)
+    return y
+
+
+def decay_memory(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w_raw: torch.Tensor, gate_raw: torch.Tensor,
+                 w_bias: torch.Tensor, bonus: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor,
+                 cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor, eps: float) -> torch.Tensor:
+    """Decayed outer-product memory read before it is written, with a bonus for the current token; state
+    [slots, H, Dk, Dv] float32 updated in place; r, k: [T, H, Dk]; v: [T, H, Dv]; w_raw [T, H * Dk]; gate_raw [T, H * Dv];
+    returns the per-head normalised, gated read-out [T, H * Dv]."""
+    dt = _dt(r, "r")
+    T, H, Dk = r.shape
+    Dv = v.shape[2]
+    for t, n in ((r, "r"), (k, "k"), (v, "v")):
+        _rows_ok(t, n)
+        _need(t.dtype == r.dtype, "r, k, v must have one dtype")
+    _need(k.shape == (T, H, Dk) and v.shape[:2] == (T, H), "r / k / v rows differ")
+    for t, n, cols in ((w_raw, "w_raw", H * Dk), (gate_raw, "gate_raw", H * Dv)):
+        _rows2d(t, n)
+        _need(t.shape == (T, cols) and t.dtype == r.dtype, f"{n} must be [T, {cols}] of r's dtype")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, Dk, Dv),
+          "state must be contiguous float32 [slots, H, Dk, Dv]")
+    _need(w_bias.numel() == H * Dk and bonus.numel() == H * Dk and norm_weight.numel() == H * Dv, "constant shapes")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    out = torch.empty((T, H * Dv), dtype=r.dtype, device=r.device)
+    dll = _lib.mixers()
+    rc = dll.nv_decay_memory(r.data_ptr(), k.data_ptr(), v.data_ptr(), r.stride(0), k.stride(0), v.stride(0),
+                             w_raw.data_ptr(), w_raw.stride(0), gate_raw.data_ptr(), gate_raw.stride(0),
+                             _f32c(w_bias, "w_bias"), _f32c(bonus, "bonus"), _f32c(norm_weight, "norm_weight"),
+                             state.data_ptr(), out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(),
+                             cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, H, Dk, Dv, float(eps), dt, _stream(r))
+    _lib.check(rc, "nv_decay_memory", dll)
+    return out
+
+
+def state_space_scan(x: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor, dt_raw: torch.Tensor, z: torch.Tensor,
+                     dt_bias: torch.Tensor, A_log: torch.Tensor, D_skip: torch.Tensor, state: torch.Tensor,
+                     cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor) -> torch.Tensor:
+    """State-space scan over a step's rows, state [slots, H, N, P] float32 updated in place; x: [T, H, P]; Bm, Cm:
+    [T, G, N]; dt_raw [T, H]; z [T, H * P]; returns y * silu(z) as float32 [T, H * P]."""
+    dt = _dt(x, "x")
+    T, H, P = x.shape
+    G, N = Bm.shape[1], Bm.shape[2]
+    for t, n in ((x, "x"), (Bm, "B"), (Cm, "C")):
+        _rows_ok(t, n)
+        _need(t.dtype == x.dtype, "x, B, C must have one dtype")
+    _need(Bm.shape == (T, G, N) and Cm.shape == (T, G, N) and H % G == 0, "B / C must be [T, G, N] with G dividing H")
+    for t, n, cols in ((dt_raw, "dt_raw", H), (z, "z", H * P)):
+        _rows2d(t, n)
+        _need(t.shape == (T, cols) and t.dtype == x.dtype, f"{n} must be [T, {cols}] of x's dtype")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, N, P),
+          "state must be contiguous float32 [slots, H, N, P]")
+    _need(dt_bias.numel() == H and A_log.numel() == H and D_skip.numel() == H, "constant shapes")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    out = torch.empty((T, H * P), dtype=torch.float32, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_state_space_scan(x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), x.stride(0), Bm.stride(0), Cm.stride(0),
+                                 dt_raw.data_ptr(), dt_raw.stride(0), z.data_ptr(), z.stride(0), _f32c(dt_bias, "dt_bias"),
+                                 _f32c(A_log, "A_log"), _f32c(D_skip, "D"), state.data_ptr(), out.data_ptr(), out.stride(0),
+                                 cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, H, G, N, P,
+                                 dt, _stream(x))
+    _lib.check(rc, "nv_state_space_scan", dll)
+    return out
+
+
+def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                    cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor) -> torch.Tensor:
+    """out[s] = h + (previous row of h - h) * mu[s]; h [T, C] (row stride free); mu [n, C] float32; state [slots, C] of
+    h's dtype carries each sequence's last row and is updated; returns [n, T, C]."""
+    dt = _dt(h, "h")
+    _rows2d(h, "h")
+    T, Cc = h.shape
+    _need(mu.dim() == 2 and mu.shape[1] == Cc, "mu must be [n, C]")
+    _need(state.is_cuda and state.dtype == h.dtype and state.is_contiguous() and state.shape[1:] == (Cc,),
+          "state must be contiguous [slots, C] of h's dtype")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    out = torch.empty((mu.shape[0], T, Cc), dtype=h.dtype, device=h.device)
+    dll = _lib.mixers()
+    rc = dll.nv_token_shift_mix(h.data_ptr(), h.stride(0), _f32c(mu, "mu"), mu.shape[0], state.data_ptr(), out.data_ptr(),
+                                cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, T, Cc, dt,
+                                _stream(h))
+    _lib.check(rc, "nv_token_shift_mix", dll)
+    return out
+
+
+def group_rms_norm(x: torch.Tensor, weight: torch.Tensor, groups: int, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Every row of x [T, C] float32 is cut into `groups` equal parts, each divided by its own root mean square; times
+    weight; result in out_dtype."""
+    _need(x.is_cuda and x.dtype == torch.float32, "x must be a float32 GPU tensor")
+    _rows2d(x, "x")
+    _need(weight.numel() == x.shape[1] and x.shape[1] % groups == 0, "weight must be [cols], groups must divide cols")
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_group_rms_norm(x.data_ptr(), x.stride(0), _f32c(weight, "weight"), y.data_ptr(), y.stride(0), _dt(y, "y"),
+                               x.shape[0], x.shape[1], int(groups), float(eps), _stream(x))
+    _lib.check(rc, "nv_group_rms_norm", dll)
+    return y
+
+
+def chunk_attn_prep_store(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm: torch.Tensor,
+                          k_norm: torch.Tensor, eps: float, freq: Optional[torch.Tensor], rot_dims: int,
+                          value_freq: torch.Tensor, slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                          v_cache: Optional[torch.Tensor]) -> torch.Tensor:
+    """RMS norm over the whole q / k rows, rotate-half rotary on the first rot_dims dimensions of every head, values
+    turned over all their dimensions, scatter of k / v into the paged cache; returns the prepared q [T, H, D]."""
+    dt = _dt(q, "q")
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _rows_ok(t, n)
+        _need(t.dtype == q.dtype, "q, k, v must have one dtype")
+    T, H, D = q.shape
+    G, Dv = k.shape[1], v.shape[2]
+    _need(k.shape == (T, G, D) and v.shape[:2] == (T, G), "k / v rows do not match q")
+    _need(q_norm.numel() == H * D and k_norm.numel() == G * D, "the norm weights span the whole q / k rows")
+    _need(positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T,
+          "positions must be a contiguous int64 [tokens] GPU tensor")
+    _need(value_freq.numel() == Dv // 2 and Dv % 2 == 0, "value_freq must hold Dv / 2 frequencies")
+    if rot_dims:
+        _need(freq is not None and freq.numel() == rot_dims // 2, "freq must hold rot_dims / 2 frequencies")
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "slot_mapping length != number of tokens")
+        _need(k_cache is not None and v_cache is not None and k_cache.is_contiguous() and v_cache.is_contiguous()
+              and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[2:] == (G, D)
+              and v_cache.shape[2:] == (G, Dv) and k_cache.shape[:2] == v_cache.shape[:2],
+              "caches must be contiguous [num_blocks, block_size, G, D] and [.., G, Dv] of q's dtype")
+    q_out = torch.empty((T, H, D), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_chunk_attn_prep_store(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0),
+                                      _f32c(q_norm, "q_norm"), _f32c(k_norm, "k_norm"), float(eps),
+                                      _f32c(freq, "freq") or None, int(rot_dims), _f32c(value_freq, "value_freq"),
+                                      positions.data_ptr(), _ptr(slot_mapping), q_out.data_ptr(), _ptr(k_cache),
+                                      _ptr(v_cache), dt, T, H, G, D, Dv, _stream(q))
+    _lib.check(rc, "nv_chunk_attn_prep_store", dll)
+    return q_out
+
+
+def chunk_sigmoid_tile_ok(D: int, Dv: int, dtype: torch.dtype) -> bool:
+    return bool(_lib.mixers().nv_attn_chunk_sigmoid_tile_ok(int(D), int(Dv), _lib.DTYPE_BF16 if dtype == _BF16 else _lib.DTYPE_F32))
+
+
+def attn_chunk_sigmoid_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                             cu_seqlens_k: torch.Tensor, block_tables: torch.Tensor, scale: float,
+                             head_bias: Optional[torch.Tensor], chunk: int, value_freq: torch.Tensor,
+                             tiles: Optional[tuple] = None, single_rows: bool = True) -> torch.Tensor:
+    """Sigmoid attention inside chunks of positions over a paged cache of rotated values (the sum is turned back by the
+    query's position); returns [T, H * Dv].  tiles: (tile_seq, tile_q0) int32 GPU tensors that cut the rows of sequences
+    with several rows into blocks of 64 for the MFMA kernel; None: every row on the one-wave-per-row kernel."""
+    dt = _dt(q, "q")
+    _rows_ok(q, "q")
+    T, H, D = q.shape
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.is_contiguous() and v_cache.is_contiguous()
+          and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[:3] == v_cache.shape[:3]
+          and k_cache.shape[3] == D, "caches must be contiguous [num_blocks, block_size, G, D | Dv] of q's dtype")
+    nb, bs, G, _ = k_cache.shape
+    Dv = v_cache.shape[3]
+    _i32(cu_seqlens_q, "cu_seqlens_q")
+    _i32(cu_seqlens_k, "cu_seqlens_k")
+    B = cu_seqlens_k.numel() - 1
+    _need(cu_seqlens_q.numel() == B + 1, "cu_seqlens_q / cu_seqlens_k length mismatch")
+    _need(block_tables.is_cuda and block_tables.dtype == torch.int32 and block_tables.dim() == 2
+          and block_tables.is_contiguous() and block_tables.shape[0] == B,
+          "block_tables must be a contiguous [B, max_blocks] int32 GPU tensor")
+    _need(head_bias is None or head_bias.numel() == H, "head_bias must be [H]")
+    _need(value_freq.numel() == Dv // 2, "value_freq must hold Dv / 2 frequencies")
+    n_tiles = 0
+    if tiles is not None:
+        _i32(tiles[0], "tile_seq")
+        _i32(tiles[1], "tile_q0")
+        n_tiles = tiles[0].numel()
+        _need(tiles[1].numel() == n_tiles, "tile tables differ in length")
+    out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_attn_chunk_sigmoid_paged(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+                                         cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), block_tables.data_ptr(), B,
+                                         block_tables.shape[1], T, H, G, D, Dv, nb, bs, float(scale),
+                                         _f32c(head_bias, "head_bias") or None, int(chunk),
+                                         _f32c(value_freq, "value_freq"), _ptr(tiles[0]) if n_tiles else None,
+                                         _ptr(tiles[1]) if n_tiles else None, n_tiles, int(bool(single_rows)), dt,
+                                         q.stride(0), out.stride(0), _stream(q))
+    _lib.check(rc, "nv_attn_chunk_sigmoid_paged", dll)
+    return out
+
+
+def moe_table_experts(h: torch.Tensor, ids: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+    """Experts chosen by a table: h [T, W]; ids [T, top] int32 (the experts of every token, distinct per row); gate_up
+    [E, 2 ff, W]; down [E, W, ff].  Expert: D (silu(G h) * (U h)).  Returns the UNWEIGHTED outputs of every token's
+    experts, [T, top, W] float32 (the stream update scales and sums them)."""
+    dt = _dt(h, "h")
+    _rows2d(h, "h")
+    T, W = h.shape
+    E, ff = gate_up.shape[0], gate_up.shape[1] // 2
+    top = ids.shape[1]
+    _need(ids.is_cuda and ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape == (T, top),
+          "ids must be contiguous int32 [T, top]")
+    _need(gate_up.is_cuda and down.is_cuda and gate_up.is_contiguous() and down.is_contiguous() and gate_up.dtype == h.dtype
+          and down.dtype == h.dtype and gate_up.shape == (E, 2 * ff, W) and down.shape == (E, W, ff),
+          "gate_up must be [E, 2 ff, W] and down [E, W, ff], contiguous, of h's dtype")
+    dll = _lib.mixers()
+    dev, P, s = h.device, T * top, _stream(h)
+    out = torch.empty((T, top, W), dtype=torch.float32, device=dev)
+    if T == 0:
+        return out
+    wgt = torch.ones((T, top), dtype=torch.float32, device=dev)
+    rows = dll.nv_moe_tile_rows(P, E)
+    tiles = dll.nv_moe_max_tiles(P, E, rows)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    meta = torch.empty(1 + 3 * tiles, dtype=torch.int32, device=dev)
+    _lib.check(dll.nv_moe_align(ids.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), P, E, rows, s), "nv_moe_align", dll)
+    y = torch.empty((P, ff), dtype=h.dtype, device=dev)
+    _lib.check(dll.nv_moe_gate_up_act(h.data_ptr(), h.stride(0), gate_up.data_ptr(), sorted_pairs.data_ptr(),
+                                      meta.data_ptr(), y.data_ptr(), dt, P, E, int(top), W, ff, float("inf"), 1.0, 0.0,
+                                      rows, s), "nv_moe_gate_up_act", dll)
+    _lib.check(dll.nv_moe_down(y.data_ptr(), down.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), wgt.data_ptr(),
+                               out.data_ptr(), dt, P, E, W, ff, rows, s), "nv_moe_down", dll)
+    return out

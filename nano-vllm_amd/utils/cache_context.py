@@ -53,6 +53,9 @@ class CacheContext:
     # Extension (optional): [B] int32, the state slot of every sequence of the step, for layers that carry a
     # recurrent state per sequence (layers/delta_rule.py).  None for models without such layers.
     state_slots: Optional[torch.Tensor] = None
+    # Extension (optional): host copy (numpy int32 [B+1]) of cu_seqlens_q, for layers that lay out their launch per
+    # sequence on the host (layers/chunk_attention.py cuts prompt portions into row tiles).
+    cu_seqlens_q_host: Optional[object] = None
 
 
 _cache_context: ContextVar[Optional[CacheContext]] = ContextVar("CacheContext", default=None)
