@@ -71,6 +71,8 @@ def embed(cfg, weights, tokens):
 # ------------------------------------------------------------------------------------------ rotary
 def rotate_halves(x, positions, dims, base, sign=1.0):
     """x [T, ..., D]: the first `dims` dimensions turn, pair (i, i + dims/2) by sign * position * base^(-2i/dims)."""
+    if dims == 0:
+        return x.float()
     half = dims // 2
     f = torch.tensor([float(base) ** (-2.0 * i / dims) for i in range(half)], dtype=torch.float32)
     ang = positions.to(torch.float32)[:, None] * f[None, :] * sign
@@ -92,7 +94,8 @@ def chunk_sigmoid_attention(m, w, p, h, eps, dtype):
     is rotated back by the query's position."""
     T = h.shape[0]
     H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
-    rot_dims, base, size = int(m["rot"]["dims"]), float(m["rot"]["base"]), int(m["mask"]["size"])
+    rot = m.get("rot") or {}
+    rot_dims, base, size = int(rot.get("dims", 0)), float(rot.get("base", 10000.0)), int((m.get("mask") or {}).get("size", 0))
     pos = torch.arange(T)
     q = rms_norm(linear(h, w[p + "q"], dtype), w[p + "q.norm"], eps).view(T, H, D)
     k = rms_norm(linear(h, w[p + "k"], dtype), w[p + "k.norm"], eps).view(T, G, D)
@@ -100,7 +103,9 @@ def chunk_sigmoid_attention(m, w, p, h, eps, dtype):
     q = rotate_halves(q, pos, rot_dims, base).to(dtype).float()
     k = rotate_halves(k, pos, rot_dims, base).to(dtype).float()
     v = rotate_halves(v, pos, Dv, base).to(dtype).float()
-    visible = (pos[None, :] <= pos[:, None]) & ((pos[None, :] // size) == (pos[:, None] // size))
+    visible = pos[None, :] <= pos[:, None]
+    if size:                                  # (no mask in the configuration: plain causal)
+        visible = visible & ((pos[None, :] // size) == (pos[:, None] // size))
     out = torch.zeros(T, H, Dv)
     for hh in range(H):
         g = hh // (H // G)
