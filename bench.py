@@ -68,6 +68,9 @@ def parse():
     ap.add_argument("--benarax", action="store_true",
                     help="instead of the default workload: the Benarax kernels and model beside Buvalix at equal sizes "
                          "(one GPU, random weights), one JSON line")
+    ap.add_argument("--divadra", action="store_true",
+                    help="instead of the default workload: the Divadra kernels and model beside Benarax at equal sizes "
+                         "(one GPU, random weights), one JSON line")
     return ap.parse_args()
 
 
@@ -799,6 +802,12 @@ def main():
             raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
         from tools.benarax_bench import run as benarax_run
         print(json.dumps(benarax_run("cuda:0")))
+        return
+    if args.divadra:
+        if not torch.cuda.is_available():
+            raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
+        from tools.divadra_bench import run as divadra_run
+        print(json.dumps(divadra_run("cuda:0")))
         return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
