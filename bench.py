@@ -70,7 +70,7 @@ def parse():
                          "(one GPU, random weights), one JSON line")
     ap.add_argument("--divadra", action="store_true",
                     help="instead of the default workload: the Divadra kernels and model beside Benarax at equal sizes "
-                         "(one GPU, random weights), one JSON line")
+                         "(one GPU, random weights), one JSON line; switched off unless NV_ALLOW_DIVADRA_BENCH=1")
     return ap.parse_args()
 
 

@@ -63,8 +63,10 @@ struct DmArgs {
     int tile;
 };
 
-template <typename T, int RPL, bool SCAN>
-__global__ void decay_memory_kernel(const DmArgs<T> a) {
+// MAXT: the most threads a launch of this instantiation has (16 value columns per wave): the register budget of the state
+// rows follows from it, so that the usual sizes (up to 128 value columns) keep the state in registers.
+template <typename T, int RPL, bool SCAN, int MAXT>
+__global__ __launch_bounds__(MAXT) void decay_memory_kernel(const DmArgs<T> a) {
     constexpr int DP = (RPL + 4) * 4;                 // LDS words per token and vector: four runs of RPL rows, padded
     extern __shared__ float smem[];
     const int tile = a.tile, Dk = a.Dk, Dv = a.Dv, H = a.H;
@@ -208,12 +210,20 @@ static int launch_decay_memory(DmArgs<T> a, int B, hipStream_t s, const char* wh
     const size_t per_token = sizeof(float) * (size_t)(3 * (rpl + 4) * 4 + 2 * a.Dv + 3);
     a.tile = (int)std::max<size_t>(1, std::min<size_t>(kDmMaxTile, kDmLdsBudget / per_token));
     const size_t smem = per_token * a.tile;
+#define NV_DM_CASE(R)                                                                                           \
+    case R:                                                                                                     \
+        if (waves <= 4) hipLaunchKernelGGL((decay_memory_kernel<T, R, SCAN, 256>), grid, block, smem, s, a);        \
+        else if (waves <= 8) hipLaunchKernelGGL((decay_memory_kernel<T, R, SCAN, 512>), grid, block, smem, s, a);   \
+        else hipLaunchKernelGGL((decay_memory_kernel<T, R, SCAN, 1024>), grid, block, smem, s, a);                  \
+        break;
     switch (rpl) {
-        case 8: hipLaunchKernelGGL((decay_memory_kernel<T, 8, SCAN>), grid, block, smem, s, a); break;
-        case 16: hipLaunchKernelGGL((decay_memory_kernel<T, 16, SCAN>), grid, block, smem, s, a); break;
-        case 32: hipLaunchKernelGGL((decay_memory_kernel<T, 32, SCAN>), grid, block, smem, s, a); break;
-        default: hipLaunchKernelGGL((decay_memory_kernel<T, 64, SCAN>), grid, block, smem, s, a); break;
+        NV_DM_CASE(8)
+        NV_DM_CASE(16)
+        NV_DM_CASE(32)
+        default:
+        NV_DM_CASE(64)
     }
+#undef NV_DM_CASE
     return check_launch(what);
 }
 
