@@ -3,7 +3,7 @@ two-norm stream boundary, squared ReLU, causal convolutions with carried inputs,
 with a bonus, the state-space scan, the grouped norm, chunked sigmoid attention over the paged cache, table-routed
 experts), with the same constructors and the same cache / state layouts as the HIP-backed modules.  They let the whole
 engine run without a GPU and give GPU tests an eager reference per layer.  Device-agnostic, slow, written from the
-layer contracts; the product model never imports it."""
+layer interfaces; the product model never imports it."""
 from __future__ import annotations
 
 import torch
