@@ -90,7 +90,8 @@ NV_API int64_t nv_attn_scoremod_workspace_bytes(int num_seqs, int64_t T, int H, 
 /*
  * Short causal convolution over time per channel, then SiLU, with the last taps-1 inputs of every sequence carried
  * in conv_state[slot] ([num_slots, taps-1, C] of dtype).  x, y: [T, C] with row strides; w: [C, taps] fp32, the
- * last column multiplies the current token.  A sequence at position 0 ignores what its slot holds.  taps <= 8.
+ * last column multiplies the current token.  A sequence at position 0 ignores what its slot holds.  taps <= 64
+ * (up to 8 the window is kept in registers).
  */
 NV_API int nv_causal_conv_silu(const void* x, int64_t x_stride, const float* w, void* conv_state, void* y,
                                int64_t y_stride, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,

@@ -159,6 +159,28 @@ __global__ __launch_bounds__(256) void causal_conv_silu_pieces_kernel(
     }
 }
 
+// More taps than the register window holds: one thread per channel walks the state rows upwards, so a row is read
+// (row s + len_q) before it is overwritten.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_walk_kernel(
+    const T* __restrict__ x, int64_t x_stride, T* __restrict__ conv_state, const int* __restrict__ cu_q,
+    const int* __restrict__ cu_k, const int* __restrict__ state_slots, int C, int taps) {
+    const int b = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int q0 = cu_q[b], nq = cu_q[b + 1] - q0, nk = cu_k[b + 1] - cu_k[b];
+    if (nq <= 0) return;
+    const int keep = taps - 1, start = nk - nq;
+    T* st = conv_state + (int64_t)state_slots[b] * keep * C;
+    for (int s = 0; s < keep; ++s) {
+        const int p = nk - keep + s;               // position this row holds afterwards
+        T v = (T)0.f;
+        if (p >= start) v = x[(int64_t)(q0 + p - start) * x_stride + c];
+        else if (p >= 0) v = st[(int64_t)(s + nq) * C + c];
+        st[(int64_t)s * C + c] = v;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_update_kernel(
     const T* __restrict__ x, int64_t x_stride, T* __restrict__ conv_state, const int* __restrict__ cu_q,
@@ -366,8 +388,8 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
                                         int taps, int dtype, void* stream) {
     using namespace nv;
     NV_REQUIRE(num_seqs >= 0 && T >= 0 && C > 0, NV_ERR_INVALID_ARG, "nv_causal_conv_silu: bad sizes");
-    NV_REQUIRE(taps >= 1 && taps <= kConvMaxTaps, NV_ERR_UNSUPPORTED, "nv_causal_conv_silu: taps=%d not in 1..%d", taps,
-               kConvMaxTaps);
+    NV_REQUIRE(taps >= 1 && taps <= 64, NV_ERR_UNSUPPORTED, "nv_causal_conv_silu: taps=%d not in 1..64", taps);
+    const bool wide = taps > kConvMaxTaps;                     // beyond the register window: the plain kernels
     if (T == 0 || num_seqs == 0) return NV_OK;
     NV_REQUIRE(x && w && y && cu_seqlens_q && cu_seqlens_k && state_slots && (conv_state || taps == 1),
                NV_ERR_INVALID_ARG, "nv_causal_conv_silu: null pointer");
@@ -376,7 +398,7 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
     hipStream_t s = (hipStream_t)stream;
     const unsigned cb = (unsigned)((C + 255) / 256);
     const int n = dtype == NV_DTYPE_BF16 ? 8 : 4;              // channels in a 16-byte piece
-    const bool pieces = C % n == 0 && x_stride % n == 0 && y_stride % n == 0 &&
+    const bool pieces = !wide && C % n == 0 && x_stride % n == 0 && y_stride % n == 0 &&
                         ((uintptr_t)x | (uintptr_t)y | (uintptr_t)conv_state) % 16 == 0;
     const unsigned pb = (unsigned)((C / n + 255) / 256);
     const int tpg = T * pb >= 8192 ? 16 : T * pb >= 2048 ? 4 : 1;      // tokens per workgroup: at least 512 workgroups
@@ -389,7 +411,11 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
         hipLaunchKernelGGL(causal_conv_silu_kernel<__bf16>, dim3((unsigned)T, cb), dim3(256), 0, s, (const __bf16*)x,
                            x_stride, w, bias, (const __bf16*)conv_state, (__bf16*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
                            state_slots, num_seqs, C, taps);
-        if (taps > 1)
+        if (wide)
+            hipLaunchKernelGGL(conv_state_walk_kernel<__bf16>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
+                               (const __bf16*)x, x_stride, (__bf16*)conv_state, cu_seqlens_q, cu_seqlens_k,
+                               state_slots, C, taps);
+        else if (taps > 1)
             hipLaunchKernelGGL(conv_state_update_kernel<__bf16>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
                                (const __bf16*)x, x_stride, (__bf16*)conv_state, cu_seqlens_q, cu_seqlens_k,
                                state_slots, C, taps);
@@ -402,7 +428,11 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
         hipLaunchKernelGGL(causal_conv_silu_kernel<float>, dim3((unsigned)T, cb), dim3(256), 0, s, (const float*)x,
                            x_stride, w, bias, (const float*)conv_state, (float*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
                            state_slots, num_seqs, C, taps);
-        if (taps > 1)
+        if (wide)
+            hipLaunchKernelGGL(conv_state_walk_kernel<float>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
+                               (const float*)x, x_stride, (float*)conv_state, cu_seqlens_q, cu_seqlens_k, state_slots,
+                               C, taps);
+        else if (taps > 1)
             hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
                                (const float*)x, x_stride, (float*)conv_state, cu_seqlens_q, cu_seqlens_k, state_slots,
                                C, taps);

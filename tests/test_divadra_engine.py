@@ -48,6 +48,7 @@ MIXED = config([parallel_layer(), mamba_layer(mlp=moe(experts=4, top=1)), parall
                 rot_dims=2, r_heads=2, r_dim=9, mlp=dense(24)), mamba_layer(heads=3, vdim=8, state=5, groups=1, norm_groups=1, conv=2, mlp=None),
                 parallel_layer(kv_heads=1, mlp=moe(experts=3, top=3, ff=10))])
 SINGLE = {"mamba2": config([mamba_layer()]),
+          "mamba2_eleven_taps": config([mamba_layer(conv=11, mlp=None)], taps=9),
           "mamba2_one_tap_conv": config([mamba_layer(conv=1, groups=4, norm_groups=4)], taps=1),
           "parallel": config([parallel_layer()]),
           "parallel_full_rotary_no_chunk": config([parallel_layer(dim=8, rot_dims=8, chunk=0, mlp=dense())], taps=5),

@@ -141,7 +141,7 @@ def test_state_space_scan_and_group_norm(dt, step, H, G, N, P):
         assert rel(hip_layers().group_rms_norm(ya, w, groups, 1e-6, dt), R.group_rms_norm(yb, w, groups, 1e-6, dt)) < tol(dt)
 
 
-@pytest.mark.parametrize("C,taps", [(96, 4), (100, 2), (1032, 3), (64, 1)])
+@pytest.mark.parametrize("C,taps", [(96, 4), (100, 2), (1032, 3), (64, 1), (96, 11), (40, 9)])
 def test_conv_bias_silu(dt, step, C, taps):
     T, _ = step
     a, b = pair("ConvBiasSilu", C, taps)
