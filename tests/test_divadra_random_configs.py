@@ -50,10 +50,10 @@ def draw_config(seed: int) -> dict:
                     "rot": {"dims": rng.choice([d for d in (2, 4, 8, 10, 16, 32, 64) if d <= dim]), "base": rng.choice([50.0, 1e4, 3e5])}}
             right = {"heads": rng.randint(1, 4), "dim": rng.choice([4, 8, 12, 16, 20, 32, 36, 64])}
             layers.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp()})
-    buckets = rng.choice([1, 2, 7, 64, 509])
+    buckets = rng.choice([1, 2, 7, 64, 211])
     return {"architecture": "Divadra", "layers": layers, "norm": {"eps": rng.choice([1e-6, 1e-5, 1e-4])},
             "vocab": rng.randint(20, 120), "width": width, "canon": {"taps": rng.randint(1, 5)},
-            "embedding": {"bigram": {"buckets": buckets, "mul_prev": rng.choice([1, 31, 127, 1000003]), "mul_cur": rng.choice([1, 7, 13])}}}
+            "embedding": {"bigram": {"buckets": buckets, "mul_prev": rng.choice([1, 31, 257, 1000003]), "mul_cur": rng.choice([1, 5, 13])}}}
 
 
 def per_position(got, want):

@@ -59,11 +59,11 @@ def pair(cls_name, *args, **kw):
     return a, b
 
 
-@pytest.mark.parametrize("W,buckets", [(96, 13), (100, 509), (2048, 7), (40, 0)])
+@pytest.mark.parametrize("W,buckets", [(96, 13), (100, 211), (2048, 7), (40, 0)])
 def test_hashed_bigram_embedding(dt, step, W, buckets):
     T, _ = step
     V = 70
-    a, b = pair("HashedBigramEmbedding", V, W, buckets, 127, 7, 1e-6, dtype=dt)
+    a, b = pair("HashedBigramEmbedding", V, W, buckets, 31, 5, 1e-6, dtype=dt)
     g = torch.Generator().manual_seed(W)
     ids = torch.randint(0, V, (T,), generator=g).to(DEV)
     pos = step[1]
@@ -153,7 +153,7 @@ def test_conv_bias_silu(dt, step, C, taps):
     assert rel(ya, yb) < tol(dt) and torch.equal(sa, sb)
 
 
-@pytest.mark.parametrize("H,G,D,Dv,chunk,rot", [(6, 3, 10, 8, 7, 6), (4, 1, 48, 48, 12, 48), (2, 2, 64, 64, 20, 32), (4, 2, 128, 64, 0, 64),
+@pytest.mark.parametrize("H,G,D,Dv,chunk,rot", [(6, 3, 10, 8, 7, 6), (4, 1, 40, 56, 12, 40), (2, 2, 64, 64, 20, 32), (4, 2, 128, 64, 0, 64),
                                                  (2, 1, 64, 128, 9, 0), (2, 2, 128, 128, 16, 128), (3, 1, 20, 130, 5, 4)])
 def test_chunk_sigmoid_attention(dt, step, H, G, D, Dv, chunk, rot):
     """Head sizes 64 / 128 in bfloat16 take the MFMA tile kernel for the rows of sequences with several rows."""
@@ -193,7 +193,7 @@ def test_chunk_sigmoid_attention_long_portions_on_the_tile_kernel(D, Dv, chunk):
         nv.set_context(None)
 
 
-@pytest.mark.parametrize("E,top,ff,W", [(5, 2, 12, 36), (16, 2, 64, 320), (40, 1, 24, 100), (3, 3, 130, 64)])
+@pytest.mark.parametrize("E,top,ff,W", [(5, 2, 12, 36), (12, 2, 48, 288), (40, 1, 24, 100), (3, 3, 130, 64)])
 def test_table_experts(dt, E, top, ff, W):
     g = torch.Generator().manual_seed(E * ff)
     V, T = 50, 61
