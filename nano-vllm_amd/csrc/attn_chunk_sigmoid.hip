@@ -17,8 +17,9 @@
 // angle = position * freq[i] as an fp32 product, full-precision sincosf), the value rotation, and the scatter of the
 // step's K/V rows into the cache.
 //
-// Two attention kernels: one wave per (query, head) in fp32 arithmetic for any element type and size (single rows,
-// float32 models), and a bf16 MFMA tile kernel for prompt portions (64 queries of one head per workgroup).
+// Two attention kernels: one wave per (query, kv head) in fp32 arithmetic for any element type and size (single rows,
+// float32 models; the heads of a group share every key and value read), and a bf16 MFMA tile kernel for prompt portions
+// (64 queries of one head per workgroup).
 #include <algorithm>
 
 #include "nv_common.h"
@@ -102,23 +103,25 @@ __global__ __launch_bounds__(256) void chunk_attn_prep_store_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------ one wave per row
-// One wave per (query token, query head).  Keys go by in tiles of 64: lane j scores key j of the tile (its own K row,
-// q broadcast from LDS), the tile's weights go through LDS, then the lanes switch to value channels (lane c accumulates
-// channels c, c + 64, ...) and stream the tile's V rows, which are contiguous per key.
+// One wave per (query token, kv head), for the REP query heads of the group at once (a group with more heads takes
+// several passes), so a cached key or value is read once per group.  Keys go by in tiles of 64: lane j scores key j of
+// the tile against every head (its own K row, the q rows broadcast from LDS), the tile's weights go through LDS, then the
+// lanes switch to value channels (lane c accumulates channels c, c + 64, ... of every head) and stream the tile's V rows,
+// which are contiguous per key.
 constexpr int kCsMaxDvPerLane = 8;   // Dv <= 512
 
-template <typename T>
+template <typename T, int REP>
 __global__ __launch_bounds__(64) void attn_chunk_sigmoid_rowwave_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     const int* __restrict__ cu_q, const int* __restrict__ cu_k, const int* __restrict__ block_tables, int B,
     int max_blocks, int H, int G, int D, int Dv, int block_size, float scale, const float* __restrict__ head_bias,
     int chunk, const float* __restrict__ vfreq, int64_t q_stride, int64_t out_stride, int only_single_rows) {
     extern __shared__ float smem[];
-    float* qs = smem;                      // [D]
-    float* ps = smem + D;                  // [64]
-    float* os = ps + 64;                   // [Dv]
-    int64_t* rows = (int64_t*)(os + Dv + ((D + Dv) & 1));   // [64] element offsets of the tile's cache rows
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    float* qs = smem;                      // [REP][D]
+    float* ps = qs + REP * D;              // [REP][64]
+    float* os = ps + REP * 64;             // [Dv]
+    int64_t* rows = (int64_t*)(os + Dv + ((REP * D + Dv) & 1));   // [64] element offsets of the tile's cache rows
+    const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
     int lo = 0, hi = B;
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -130,54 +133,87 @@ __global__ __launch_bounds__(64) void attn_chunk_sigmoid_rowwave_kernel(
     if ((only_single_rows == 1 && len_q != 1) || (only_single_rows == 2 && len_q == 1)) return;
     const int pos = len_k - len_q + (t - cu_q[b]);      // this query's position
     const int first = chunk > 0 ? (pos / chunk) * chunk : 0;     // it sees keys first .. pos
-    const int g = h / (H / G);
-    for (int d = lane; d < D; d += 64) qs[d] = (float)q[(int64_t)t * q_stride + (int64_t)h * D + d];
+    const int per = H / G, vh = Dv / 2;
     const int* table = block_tables + (int64_t)b * max_blocks;
-    const float hb = head_bias ? head_bias[h] : 0.f;
-    float acc[kCsMaxDvPerLane] = {};
-    __syncthreads();
-    for (int base = first; base <= pos; base += 64) {
-        const int j = base + lane;
-        float p = 0.f;
-        int64_t row = 0;
-        if (j <= pos) {
-            const int blk = table[j / block_size];
-            row = ((int64_t)blk * block_size + (j % block_size)) * G + g;
-            const T* kr = k_cache + row * D;
-            float dot = 0.f;
-            for (int d = 0; d < D; ++d) dot += qs[d] * (float)kr[d];
-            p = 1.0f / (1.0f + expf(-(dot * scale + hb)));
-        }
-        __syncthreads();                                     // previous tile's readers are done
-        ps[lane] = p;
-        rows[lane] = row;
+    for (int h0 = 0; h0 < per; h0 += REP) {
+        const int n = min(REP, per - h0);                // heads of this pass: g * per + h0 .. + n - 1
+        __syncthreads();                                 // the previous pass is done with qs, ps, os
+        for (int i = lane; i < n * D; i += 64)
+            qs[i] = (float)q[(int64_t)t * q_stride + (int64_t)(g * per + h0) * D + i];
+        float hb[REP];
+#pragma unroll
+        for (int r = 0; r < REP; ++r) hb[r] = (head_bias && r < n) ? head_bias[g * per + h0 + r] : 0.f;
+        float acc[REP][kCsMaxDvPerLane] = {};
         __syncthreads();
-        const int n_tile = min(64, pos + 1 - base);
-        for (int jj = 0; jj < n_tile; ++jj) {
-            const float pj = ps[jj];
-            const T* vr = v_cache + rows[jj] * Dv;
+        for (int base = first; base <= pos; base += 64) {
+            const int j = base + lane;
+            float dot[REP] = {};
+            int64_t row = 0;
+            if (j <= pos) {
+                const int blk = table[j / block_size];
+                row = ((int64_t)blk * block_size + (j % block_size)) * G + g;
+                const T* kr = k_cache + row * D;
+                for (int d = 0; d < D; ++d) {
+                    const float kd = (float)kr[d];
+#pragma unroll
+                    for (int r = 0; r < REP; ++r) dot[r] += qs[r * D + d] * kd;      // (rows past n hold stale, finite values)
+                }
+            }
+            __syncthreads();                                     // previous tile's readers are done
+#pragma unroll
+            for (int r = 0; r < REP; ++r) ps[r * 64 + lane] = (j <= pos && r < n) ? 1.0f / (1.0f + expf(-(dot[r] * scale + hb[r]))) : 0.f;
+            rows[lane] = row;
+            __syncthreads();
+            const int n_tile = min(64, pos + 1 - base);
+            for (int jj = 0; jj < n_tile; ++jj) {
+                const T* vr = v_cache + rows[jj] * Dv;
+#pragma unroll
+                for (int i = 0; i < kCsMaxDvPerLane; ++i) {
+                    const int c = lane + 64 * i;
+                    if (c < Dv) {
+                        const float vv = (float)vr[c];
+#pragma unroll
+                        for (int r = 0; r < REP; ++r) acc[r][i] += ps[r * 64 + jj] * vv;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < REP; ++r) {
+            if (r >= n) break;
+            __syncthreads();                                     // the previous head's pairs have been read
 #pragma unroll
             for (int i = 0; i < kCsMaxDvPerLane; ++i) {
                 const int c = lane + 64 * i;
-                if (c < Dv) acc[i] += pj * (float)vr[c];
+                if (c < Dv) os[c] = acc[r][i];
+            }
+            __syncthreads();
+            T* dst = out + (int64_t)t * out_stride + (int64_t)(g * per + h0 + r) * Dv;
+            for (int m = lane; m < vh; m += 64) {
+                const float a = os[m], bb = os[m + vh];
+                float sn, cs;
+                sincosf((float)pos * vfreq[m], &sn, &cs);        // turned back: angle -pos * f
+                dst[m] = (T)(a * cs + bb * sn);
+                dst[m + vh] = (T)(bb * cs - a * sn);
             }
         }
     }
-#pragma unroll
-    for (int i = 0; i < kCsMaxDvPerLane; ++i) {
-        const int c = lane + 64 * i;
-        if (c < Dv) os[c] = acc[i];
-    }
-    __syncthreads();
-    const int vh = Dv / 2;
-    for (int m = lane; m < vh; m += 64) {
-        const float a = os[m], bb = os[m + vh];
-        float sn, cs;
-        sincosf((float)pos * vfreq[m], &sn, &cs);            // turned back: angle -pos * f
-        T* dst = out + (int64_t)t * out_stride + (int64_t)h * Dv;
-        dst[m] = (T)(a * cs + bb * sn);
-        dst[m + vh] = (T)(bb * cs - a * sn);
-    }
+}
+
+template <typename T>
+static void launch_cs_rowwave(int rep, dim3 grid, hipStream_t s, const T* q, const T* kc, const T* vc, T* out, const int* cu_q,
+                              const int* cu_k, const int* bt, int B, int max_blocks, int H, int G, int D, int Dv, int block_size,
+                              float scale, const float* hb, int chunk, const float* vfreq, int64_t q_stride, int64_t out_stride,
+                              int mode) {
+    const size_t smem = sizeof(float) * (size_t)(rep * D + rep * 64 + Dv + ((rep * D + Dv) & 1)) + sizeof(int64_t) * 64;
+#define NV_CS_ROW(R)                                                                                                       \
+    hipLaunchKernelGGL((attn_chunk_sigmoid_rowwave_kernel<T, R>), grid, dim3(64), smem, s, q, kc, vc, out, cu_q, cu_k, bt, B, \
+                       max_blocks, H, G, D, Dv, block_size, scale, hb, chunk, vfreq, q_stride, out_stride, mode)
+    if (rep == 1) NV_CS_ROW(1);
+    else if (rep == 2) NV_CS_ROW(2);
+    else if (rep == 4) NV_CS_ROW(4);
+    else NV_CS_ROW(8);
+#undef NV_CS_ROW
 }
 
 // ------------------------------------------------------------------------------------------------ prompt portions
@@ -413,16 +449,20 @@ extern "C" int nv_attn_chunk_sigmoid_paged(const void* q, const void* k_cache, c
         if (single_rows == 0) return NV_OK;                 // the step has no single rows
         rowwave_mode = 1;
     }
-    const size_t smem = sizeof(float) * (size_t)(D + 64 + Dv + ((D + Dv) & 1)) + sizeof(int64_t) * 64;
+    // query heads taken per pass: the group's, rounded up to 1, 2, 4 or 8; fewer when the q rows would not fit into LDS
+    const int per = H / G;
+    int rep = per <= 1 ? 1 : per <= 2 ? 2 : per <= 4 ? 4 : 8;
+    while (rep > 1 && sizeof(float) * (size_t)rep * (D + 64) > 40 * 1024) rep /= 2;
+    NV_REQUIRE(sizeof(float) * (size_t)(D + 64 + Dv + 1) + 512 <= 60 * 1024, NV_ERR_UNSUPPORTED,
+               "nv_attn_chunk_sigmoid_paged: key size %d too large", D);
+    const dim3 grid((unsigned)T, (unsigned)G);
     if (dtype == NV_DTYPE_BF16)
-        hipLaunchKernelGGL(attn_chunk_sigmoid_rowwave_kernel<__bf16>, dim3((unsigned)T, (unsigned)H), dim3(64), smem, s,
-                           (const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q,
-                           cu_seqlens_k, block_tables, num_seqs, max_blocks, H, G, D, Dv, block_size, scale, head_bias,
-                           chunk, value_freq, q_stride, out_stride, rowwave_mode);
+        launch_cs_rowwave<__bf16>(rep, grid, s, (const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out,
+                                  cu_seqlens_q, cu_seqlens_k, block_tables, num_seqs, max_blocks, H, G, D, Dv, block_size, scale,
+                                  head_bias, chunk, value_freq, q_stride, out_stride, rowwave_mode);
     else
-        hipLaunchKernelGGL(attn_chunk_sigmoid_rowwave_kernel<float>, dim3((unsigned)T, (unsigned)H), dim3(64), smem, s,
-                           (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out, cu_seqlens_q,
-                           cu_seqlens_k, block_tables, num_seqs, max_blocks, H, G, D, Dv, block_size, scale, head_bias,
-                           chunk, value_freq, q_stride, out_stride, rowwave_mode);
+        launch_cs_rowwave<float>(rep, grid, s, (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out,
+                                 cu_seqlens_q, cu_seqlens_k, block_tables, num_seqs, max_blocks, H, G, D, Dv, block_size, scale,
+                                 head_bias, chunk, value_freq, q_stride, out_stride, rowwave_mode);
     return check_launch("nv_attn_chunk_sigmoid_paged");
 }
