@@ -154,7 +154,7 @@ def test_conv_bias_silu(dt, step, C, taps):
 
 
 @pytest.mark.parametrize("H,G,D,Dv,chunk,rot", [(6, 3, 10, 8, 7, 6), (4, 1, 40, 56, 12, 40), (2, 2, 64, 64, 20, 32), (4, 2, 128, 64, 0, 64),
-                                                 (2, 1, 64, 128, 9, 0), (2, 2, 128, 128, 16, 128), (3, 1, 20, 130, 5, 4)])
+                                                 (2, 1, 64, 128, 9, 0), (2, 2, 128, 128, 16, 128), (3, 1, 20, 130, 5, 4), (18, 2, 16, 12, 7, 8), (16, 1, 64, 64, 0, 64)])
 def test_chunk_sigmoid_attention(dt, step, H, G, D, Dv, chunk, rot):
     """Head sizes 64 / 128 in bfloat16 take the MFMA tile kernel for the rows of sequences with several rows."""
     T, pos = step
