@@ -29,7 +29,7 @@ def test_second_library_header_prototypes_and_exports_agree():
     # argument errors are reported before any device access
     assert dll.nv_add_layernorm(None, None, 0, 0, None, None, None, None, None, None, 0, 4, 64, 1e-5, None) == -1
     assert b"null residual" in dll.nv_last_error()
-    assert dll.nv_causal_conv_silu(None, 0, None, None, None, 0, None, None, None, 1, 4, 8, 9, 0, None) == -2
+    assert dll.nv_causal_conv_silu(None, 0, None, None, None, 0, None, None, None, 1, 4, 8, 65, 0, None) == -2
     assert dll.nv_gated_delta_rule(None, None, None, 0, 0, 0, None, 0, None, 0, None, 0, None, None, None, None, None,
                                    0, None, None, None, 0, 2, 2, 8, 8, 1e-5, 0, None) == 0       # no sequences: a no-op
 
