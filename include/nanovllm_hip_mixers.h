@@ -210,6 +210,14 @@ NV_API int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const float
                                     const int32_t* state_slots, int num_seqs, int64_t T, int C, int taps, int dtype,
                                     void* stream);
 
+/* The same convolution with the activation as an argument: NV_CONV_ACT_NONE leaves the sum as it is. */
+#define NV_CONV_ACT_NONE 0
+#define NV_CONV_ACT_SILU 1
+NV_API int nv_causal_conv_act(const void* x, int64_t x_stride, const float* w, const float* bias, void* conv_state,
+                              void* y, int64_t y_stride, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                              const int32_t* state_slots, int num_seqs, int64_t T, int C, int taps, int act, int dtype,
+                              void* stream);
+
 /* nv_moe_gate_up with a free shift of the up branch: act = g * sigmoid(alpha g) * (u + up_shift); limit = +inf, alpha = 1,
  * up_shift = 0 is the plain SiLU-gated unit. */
 NV_API int nv_moe_gate_up_act(const void* h, int64_t h_stride, const void* gate_up, const int32_t* sorted_pairs,
@@ -220,7 +228,7 @@ NV_API int nv_moe_gate_up_act(const void* h, int64_t h_stride, const void* gate_
  * Embedding with a hashed bigram table, RMS-normed into an fp32 stream x [T, cols]:
  *   x[t] = rmsnorm(embed[id_t] + bigram[row_t]) * norm_w,  row_t = (id_{t-1} * mul_prev + id_t * mul_cur) mod buckets,
  *   or row `buckets` at position 0.  prev_state [num_slots] int64 carries each sequence's last id between steps.
- *   bigram NULL: the embedding row alone.  embed: [vocab, cols], bigram: [buckets + 1, cols] of dtype.
+ *   bigram NULL: the embedding row alone.  norm_w NULL: the sum goes into the stream as it is.  embed: [vocab, cols], bigram: [buckets + 1, cols] of dtype.
  */
 NV_API int nv_hashed_bigram_embed(const int64_t* ids, const int64_t* positions, const void* embed, const void* bigram,
                                   int64_t buckets, int64_t mul_prev, int64_t mul_cur, const float* norm_w, float eps,
@@ -315,6 +323,81 @@ NV_API int nv_attn_chunk_sigmoid_paged(const void* q, const void* k_cache, const
                                        const float* head_bias, int chunk, const float* value_freq,
                                        const int32_t* tile_seq, const int32_t* tile_q0, int num_tiles, int single_rows,
                                        int dtype, int64_t q_stride, int64_t out_stride, void* stream);
+
+/* -------------------------------------------------------------------------------------------------
+ * An fp32 stream whose sublayers run one after the other, each output scaled per column; memories that are written
+ * before they are read; attention whose values are its un-normed keys; sigmoid routing over groups of experts.
+ * ------------------------------------------------------------------------------------------------- */
+/*
+ * One sublayer boundary of a pre-norm fp32 stream, per row and in place (every part optional):
+ *   r += col_scale * (add1 + sigmoid(gate2[row]) * add2 + sum_j parts[:, j])
+ *   y32 / y = r / sqrt(mean(r^2) + eps) * norm_w                       (fp32 and / or dtype; norm_w NULL: no norm)
+ * add1, add2: [rows, cols] of dtype with row strides; gate2: one raw gate per row of dtype, gate2_stride elements apart
+ * (NULL: add2 counts fully); parts: [rows, n_parts, cols] fp32; col_scale, norm_w: [cols] fp32.  cols <= 16384.
+ */
+NV_API int nv_stream_boundary_scaled(void* resid, const void* add1, int64_t add1_stride, const void* add2,
+                                     int64_t add2_stride, const void* gate2, int64_t gate2_stride, const float* parts,
+                                     int n_parts, const float* col_scale, const float* norm_w, float eps, float* y32,
+                                     void* y, int dtype, int64_t rows, int cols, void* stream);
+
+/* y = c0 z / rms(z) + c1 z^2 / rms(z^2) + c2 z^3 / rms(z^3) + c3 per row (powers element by element, rms(u) =
+ * sqrt(mean(u^2) + eps) over the row, fp32); x: [rows, cols] of dtype with a row stride, coef: 4 fp32 on the device,
+ * y contiguous. */
+NV_API int nv_poly_norm(const void* x, int64_t x_stride, const float* coef, float eps, void* y, int dtype, int64_t rows,
+                        int cols, void* stream);
+
+/*
+ * In front of nv_attn_scoremod_paged: per-head RMS norm of q and k (weights q_norm, k_norm [D], shared by the heads),
+ * rotate-half rotary on the first rot_dims dimensions (pair (i, i + rot_dims / 2) by positions[t] * freq[i]); the
+ * prepared k rows are scattered into k_cache and the k rows AS GIVEN into v_cache (slot < 0 or NULL mapping: skipped).
+ * q: [T, H, D], k: [T, G, D] with token strides; q_out: [T, H, D] contiguous; caches [num_slots, G, D].
+ */
+NV_API int nv_head_norm_rope_store(const void* q, const void* k, int64_t q_stride, int64_t k_stride, const float* q_norm,
+                                   const float* k_norm, float eps, const float* freq, int rot_dims,
+                                   const int64_t* positions, const int32_t* slot_mapping, void* q_out, void* k_cache,
+                                   void* v_cache, int dtype, int64_t T, int H, int G, int D, void* stream);
+
+/*
+ * Matrix memory with exponential gates, written before it is read; per slot the state [H, Dk, Dv], the normaliser
+ * [H, Dk] and the running maximum [H], all fp32 (a sequence at position 0 starts from zeros, the maximum from 0):
+ *   i = cap tanh((i_pre + i_bias) / cap);  f = logsigmoid(cap tanh((f_pre + f_bias) / cap));  m' = max(f + m, i)
+ *   S <- exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k alone;  o = S^T (q q_scale) / (max(|n . q q_scale|,
+ *   exp(-m')) + 1e-6);  out[t, h] = o / sqrt(mean(o^2) + eps) * norm_w[h] * sigmoid(gate_raw[t, h])
+ * q, k: [T, H * Dk]; v, gate_raw, out: [T, H * Dv] of dtype with token strides; i_pre, f_pre: [T, H] fp32,
+ * gate_pre_stride floats apart per token; i_bias, f_bias: [H]; norm_w: [H * Dv] fp32.  Dk, Dv <= 256.
+ */
+NV_API int nv_mlstm_memory(const void* q, const void* k, const void* v, int64_t q_stride, int64_t k_stride,
+                           int64_t v_stride, const float* i_pre, const float* f_pre, int64_t gate_pre_stride,
+                           const void* gate_raw, int64_t gate_stride, const float* i_bias, const float* f_bias,
+                           const float* norm_w, float* state, float* norm_state, float* max_state, void* out,
+                           int64_t out_stride, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                           const int32_t* state_slots, int num_seqs, int H, int Dk, int Dv, float eps, float gate_cap,
+                           float q_scale, int dtype, void* stream);
+
+/*
+ * Keyless gated linear recurrence (what is written is one minus the forget gate); state [num_slots, H, Dk, Dv] fp32:
+ *   f = lower + (1 - lower) sigmoid(f_raw + f_bias);  S <- diag(f) S + (1 - f) v^T;  o = S^T silu(q)
+ *   out[t, h] = o / sqrt(mean(o^2) + eps) * norm_w            (norm_w: [Dv], the same for every head)
+ * q, f_raw: [T, H * Dk]; v, out: [T, H * Dv] of dtype with token strides; f_bias, lower: [H * Dk] fp32.  Dk, Dv <= 256.
+ */
+NV_API int nv_gated_write_memory(const void* q, const void* f_raw, const void* v, int64_t q_stride, int64_t f_stride,
+                                 int64_t v_stride, const float* f_bias, const float* lower, const float* norm_w,
+                                 float* state, void* out, int64_t out_stride, const int32_t* cu_seqlens_q,
+                                 const int32_t* cu_seqlens_k, const int32_t* state_slots, int num_seqs, int H, int Dk,
+                                 int Dv, float eps, int dtype, void* stream);
+
+/*
+ * Routing by sigmoid scores: s = sigmoid(logits); the choice is made on s + correction (NULL: s) among the experts of
+ * the keep_groups best of n_groups equal consecutive blocks of experts (a block's merit: the sum of its top two biased
+ * scores, or its one score); weights = s of the chosen, as they are.  E <= 512.  ids, weights: [T, top].
+ */
+NV_API int nv_moe_route_grouped(const float* logits, const float* correction, int32_t* ids, float* weights, int64_t T,
+                                int E, int top, int n_groups, int keep_groups, void* stream);
+
+/* nv_moe_gate_up for experts without a gate: y[position] = max(U_e h, 0)^2, up: [E, ff, width]. */
+NV_API int nv_moe_up_relu2(const void* h, int64_t h_stride, const void* up, const int32_t* sorted_pairs,
+                           const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width, int ff,
+                           int tile_rows, void* stream);
 
 #ifdef __cplusplus
 }

@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip.so")
 MIXERS_LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip_mixers.so")
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -116,6 +116,19 @@ MIXERS_PROTOTYPES = {
     "nv_attn_chunk_sigmoid_paged": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i32, _i32,
                                            _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _i64,
                                            _vp]),
+    "nv_causal_conv_act": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32,
+                                  _vp]),
+    "nv_stream_boundary_scaled": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i32, _vp, _vp, _f32, _vp, _vp, _i32,
+                                         _i64, _i32, _vp]),
+    "nv_poly_norm": (_i32, [_vp, _i64, _vp, _f32, _vp, _i32, _i64, _i32, _vp]),
+    "nv_head_norm_rope_store": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _f32, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32,
+                                       _i64, _i32, _i32, _i32, _vp]),
+    "nv_mlstm_memory": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp,
+                               _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _i32, _vp]),
+    "nv_gated_write_memory": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i32,
+                                     _i32, _i32, _i32, _f32, _i32, _vp]),
+    "nv_moe_route_grouped": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "nv_moe_up_relu2": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
 }
 DTYPE_BF16, DTYPE_F32 = 0, 1
 

@@ -39,7 +39,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const float* __restrict__ bias,
     const T* __restrict__ conv_state, T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q,
-    const int* __restrict__ cu_k, const int* __restrict__ state_slots, int B, int C, int taps) {
+    const int* __restrict__ cu_k, const int* __restrict__ state_slots, int B, int C, int taps, int act) {
     const int t = blockIdx.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= C) return;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
         else if (start + src >= 0) xv = (float)st[(int64_t)(taps - 1 + src) * C + c];
         acc += w[(int64_t)c * taps + (taps - 1 - j)] * xv;
     }
-    y[(int64_t)t * y_stride + c] = (T)silu_f(acc);
+    y[(int64_t)t * y_stride + c] = (T)(act ? silu_f(acc) : acc);
 }
 
 // The same in 16-byte pieces: a thread takes 8 (bf16) or 4 (fp32) neighbouring channels of one token.
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_pieces_kernel(
     const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const float* __restrict__ bias,
     const T* __restrict__ conv_state, T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q,
     const int* __restrict__ cu_k, const int* __restrict__ state_slots, int B, int C, int taps, int T_rows,
-    int tokens_per_group) {
+    int tokens_per_group, int act) {
     constexpr int N = Piece<T>::n;
     const int c = (blockIdx.y * 256 + threadIdx.x) * N;
     if (c >= C) return;
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_pieces_kernel(
             for (int e = 0; e < N; ++e) acc[e] += wt[j][e] * win[j][e];       // wt[j] = 0 for j >= taps
         }
 #pragma unroll
-        for (int e = 0; e < N; ++e) acc[e] = silu_f(acc[e]);
+        for (int e = 0; e < N; ++e) acc[e] = act ? silu_f(acc[e]) : acc[e];
         Piece<T>::store(y + (int64_t)t * y_stride + c, acc);
 #pragma unroll
         for (int j = kConvMaxTaps - 1; j > 0; --j) {
@@ -386,7 +386,16 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
                                         void* conv_state, void* y, int64_t y_stride, const int* cu_seqlens_q,
                                         const int* cu_seqlens_k, const int* state_slots, int num_seqs, int64_t T, int C,
                                         int taps, int dtype, void* stream) {
+    return nv_causal_conv_act(x, x_stride, w, bias, conv_state, y, y_stride, cu_seqlens_q, cu_seqlens_k, state_slots,
+                              num_seqs, T, C, taps, NV_CONV_ACT_SILU, dtype, stream);
+}
+
+extern "C" int nv_causal_conv_act(const void* x, int64_t x_stride, const float* w, const float* bias, void* conv_state,
+                                  void* y, int64_t y_stride, const int* cu_seqlens_q, const int* cu_seqlens_k,
+                                  const int* state_slots, int num_seqs, int64_t T, int C, int taps, int act, int dtype,
+                                  void* stream) {
     using namespace nv;
+    NV_REQUIRE(act == NV_CONV_ACT_NONE || act == NV_CONV_ACT_SILU, NV_ERR_INVALID_ARG, "nv_causal_conv_act: bad activation");
     NV_REQUIRE(num_seqs >= 0 && T >= 0 && C > 0, NV_ERR_INVALID_ARG, "nv_causal_conv_silu: bad sizes");
     NV_REQUIRE(taps >= 1 && taps <= 64, NV_ERR_UNSUPPORTED, "nv_causal_conv_silu: taps=%d not in 1..64", taps);
     const bool wide = taps > kConvMaxTaps;                     // beyond the register window: the plain kernels
@@ -406,11 +415,11 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
         if (pieces)
             hipLaunchKernelGGL(causal_conv_silu_pieces_kernel<__bf16>, dim3((unsigned)((T + tpg - 1) / tpg), pb), dim3(256), 0, s,
                                (const __bf16*)x, x_stride, w, bias, (const __bf16*)conv_state, (__bf16*)y, y_stride,
-                               cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg);
+                               cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg, act);
         else
         hipLaunchKernelGGL(causal_conv_silu_kernel<__bf16>, dim3((unsigned)T, cb), dim3(256), 0, s, (const __bf16*)x,
                            x_stride, w, bias, (const __bf16*)conv_state, (__bf16*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
-                           state_slots, num_seqs, C, taps);
+                           state_slots, num_seqs, C, taps, act);
         if (wide)
             hipLaunchKernelGGL(conv_state_walk_kernel<__bf16>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
                                (const __bf16*)x, x_stride, (__bf16*)conv_state, cu_seqlens_q, cu_seqlens_k,
@@ -423,11 +432,11 @@ extern "C" int nv_causal_conv_bias_silu(const void* x, int64_t x_stride, const f
         if (pieces)
             hipLaunchKernelGGL(causal_conv_silu_pieces_kernel<float>, dim3((unsigned)((T + tpg - 1) / tpg), pb), dim3(256), 0, s,
                                (const float*)x, x_stride, w, bias, (const float*)conv_state, (float*)y, y_stride,
-                               cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg);
+                               cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg, act);
         else
         hipLaunchKernelGGL(causal_conv_silu_kernel<float>, dim3((unsigned)T, cb), dim3(256), 0, s, (const float*)x,
                            x_stride, w, bias, (const float*)conv_state, (float*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
-                           state_slots, num_seqs, C, taps);
+                           state_slots, num_seqs, C, taps, act);
         if (wide)
             hipLaunchKernelGGL(conv_state_walk_kernel<float>, dim3((unsigned)num_seqs, cb), dim3(256), 0, s,
                                (const float*)x, x_stride, (float*)conv_state, cu_seqlens_q, cu_seqlens_k, state_slots,

@@ -84,6 +84,67 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
+// Sigmoid scores with a selection bias and a choice limited to the best consecutive blocks of experts.  One wave per
+// token: the biased scores go to LDS, a lane adds up the top two of its block, every group counts how many
+// groups beat it (larger merit, then lower index) and is open when fewer than `keep` do; the choice is the wave-wide
+// arg-max of nv_moe_route over the experts of open groups, and the weights are the plain sigmoids of the chosen.
+constexpr int kMoeGroupedMaxE = 512;
+__global__ __launch_bounds__(64) void moe_route_grouped_kernel(const float* __restrict__ logits, const float* __restrict__ corr,
+                                                               int* __restrict__ ids, float* __restrict__ wgt, int E, int top,
+                                                               int n_groups, int keep) {
+    __shared__ float choice[kMoeGroupedMaxE];
+    __shared__ float merit[kMoeGroupedMaxE];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float* z = logits + t * E;
+    const int gs = E / n_groups;
+    for (int e = lane; e < E; e += 64) {
+        const float s = 1.0f / (1.0f + expf(-z[e]));
+        choice[e] = corr != nullptr ? s + corr[e] : s;
+    }
+    __syncthreads();
+    if (n_groups > 1) {
+        for (int g = lane; g < n_groups; g += 64) {
+            float a = -INFINITY, b = -INFINITY;                // the largest and the second largest of the group
+            for (int i = 0; i < gs; ++i) {
+                const float c = choice[g * gs + i];
+                if (c > a) { b = a; a = c; } else if (c > b) b = c;
+            }
+            merit[g] = gs > 1 ? a + b : a;
+        }
+        __syncthreads();
+        for (int g = lane; g < n_groups; g += 64) {
+            const float mine = merit[g];
+            int ahead = 0;
+            for (int o = 0; o < n_groups; ++o) ahead += (merit[o] > mine || (merit[o] == mine && o < g)) ? 1 : 0;
+            if (ahead >= keep)
+                for (int i = 0; i < gs; ++i) choice[g * gs + i] = -INFINITY;
+        }
+        __syncthreads();
+    }
+    unsigned taken = 0;
+    for (int j = 0; j < top; ++j) {
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+        for (int i = 0; i < kMoeGroupedMaxE / 64; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && !((taken >> i) & 1u) && (be == 0x7fffffff || choice[e] > bv)) { bv = choice[e]; be = e; }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(bv, off);
+            const int oe = __shfl_xor(be, off);
+            const bool mine_valid = be != 0x7fffffff, other_valid = oe != 0x7fffffff;
+            if (other_valid && (!mine_valid || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
+        }
+        if ((be & 63) == lane) taken |= 1u << (be >> 6);
+        if (lane == 0) {
+            ids[t * top + j] = be;
+            wgt[t * top + j] = 1.0f / (1.0f + expf(-z[be]));
+        }
+    }
+}
+
 // One workgroup.  meta: [0] = number of tiles, then (expert, first position, rows) per tile.
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int* __restrict__ sorted_pairs,
                                                          int* __restrict__ meta, int64_t P, int E, int tile_rows) {
@@ -141,20 +202,23 @@ __device__ __forceinline__ uint4 moe_fetch(const T* row, int k0, int K, bool vec
     return *(const uint4*)tmp;
 }
 
-// GATE_UP: A rows are gathered token rows, B holds the expert's gate rows and up rows, the epilogue is the activation.
-// else:    A rows are the sorted activation rows, B the expert's down rows, the epilogue weights and scatters.
+// MODE 1 (gate and up): A rows are gathered token rows, B holds the expert's gate rows and up rows, the epilogue is the
+//         gated activation.
+// MODE 2 (up alone):   A rows are gathered token rows, B the expert's up rows, the epilogue is max(x, 0)^2.
+// MODE 0 (down):       A rows are the sorted activation rows, B the expert's down rows, the epilogue weights and scatters.
 // The slices of the next step are fetched into registers while the current ones are multiplied out of LDS.
-template <typename T, int MT, int NT, bool GATE_UP>
+template <typename T, int MT, int NT, int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, const int* __restrict__ sorted_pairs,
     const int* __restrict__ meta, const float* __restrict__ pair_w, T* __restrict__ y, float* __restrict__ out, int top,
     int N, int K, float limit, float alpha, float up_shift, int vec_ok, int max_tiles) {
     using M = MoeMma<T>;
+    constexpr bool GATE_UP = MODE == 1, GATHER = MODE != 0;
     constexpr int BK = M::kBK, BM = 16 * MT, BN = 64 * NT, NB = GATE_UP ? 2 : 1, LD = BK + M::kPad, KV = BK / M::kVec;
     constexpr int A_IT = (BM * KV + 255) / 256, B_IT = (NB * BN * KV + 255) / 256;
     __shared__ __attribute__((aligned(16))) T As[BM * LD];
     __shared__ __attribute__((aligned(16))) T Bs[NB * BN * LD];
-    __shared__ int src_row[BM];                    // GATE_UP: token of the row; else the pair of the row; -1 past the tile
+    __shared__ int src_row[BM];                    // gathered rows: token of the row; else the pair of the row; -1 past the tile
     // Workgroups go to the chip's 8 XCDs (each with its own L2) round robin by their index: index i runs item
     // (i % 8) * (items / 8) + i / 8, so one XCD works through neighbouring row tiles -- the tiles of one expert, which
     // share their weight slices in that L2.  Items: row tile fastest, then the column block.
@@ -167,7 +231,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lq = lane & 15, lg = lane >> 4;
     for (int i = tid; i < BM; i += 256) {
         const int pair = i < rows ? sorted_pairs[row0 + i] : -1;
-        src_row[i] = pair < 0 ? -1 : (GATE_UP ? pair / top : pair);
+        src_row[i] = pair < 0 ? -1 : (GATHER ? pair / top : pair);
     }
     __syncthreads();
     const T* we = w + (int64_t)e * (NB * (int64_t)N) * K;     // [NB * N, K] of this expert
@@ -178,7 +242,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     for (int i = 0; i < A_IT; ++i) {
         const int it = tid + 256 * i, r = it / KV;
         a_row[i] = nullptr;
-        if (it < BM * KV && r < rows) a_row[i] = GATE_UP ? a + (int64_t)src_row[r] * a_stride : a + (int64_t)(row0 + r) * a_stride;
+        if (it < BM * KV && r < rows) a_row[i] = GATHER ? a + (int64_t)src_row[r] * a_stride : a + (int64_t)(row0 + r) * a_stride;
     }
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
@@ -236,6 +300,9 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
                     const float g = fminf(acc[nt][m][i], limit);
                     const float u = fminf(fmaxf(acc[NT + nt][m][i], -limit), limit);
                     y[(int64_t)(row0 + r) * N + n] = (T)(g / (1.0f + expf(-alpha * g)) * (u + up_shift));
+                } else if constexpr (MODE == 2) {
+                    const float u = fmaxf(acc[nt][m][i], 0.f);
+                    y[(int64_t)(row0 + r) * N + n] = (T)(u * u);
                 } else {
                     const int pair = src_row[r];
                     out[(int64_t)pair * N + n] = acc[nt][m][i] * pair_w[pair];
@@ -245,7 +312,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     }
 }
 
-template <typename T, bool GATE_UP>
+template <typename T, int MODE>
 static void launch_grouped(const void* a, int64_t a_stride, const void* w, const int* sorted_pairs, const int* meta,
                            const float* pair_w, void* y, float* out, int top, int N, int K, float limit, float alpha,
                            float up_shift, int max_tiles, int tile_rows, hipStream_t s) {
@@ -254,7 +321,7 @@ static void launch_grouped(const void* a, int64_t a_stride, const void* w, const
     // many rows per expert: 64 x 128 tiles (a wave owns 32 columns; 128-row tiles measured slower: one workgroup per CU);
     // few: 16 x 64 tiles, more workgroups per weight byte
 #define NV_MOE_LAUNCH(MT, NT)                                                                                          \
-    hipLaunchKernelGGL((moe_grouped_kernel<T, MT, NT, GATE_UP>), dim3((unsigned)(max_tiles * ((N + 64 * NT - 1) / (64 * NT)))), \
+    hipLaunchKernelGGL((moe_grouped_kernel<T, MT, NT, MODE>), dim3((unsigned)(max_tiles * ((N + 64 * NT - 1) / (64 * NT)))), \
                        dim3(256), 0, s, (const T*)a, a_stride, (const T*)w, sorted_pairs, meta, pair_w, (T*)y, out, top, N, K,  \
                        limit, alpha, up_shift, vec_ok, max_tiles)
     if (tile_rows == 64 && sizeof(T) == 2) NV_MOE_LAUNCH(4, 2);
@@ -315,10 +382,10 @@ extern "C" int nv_moe_gate_up_act(const void* h, int64_t h_stride, const void* g
     NV_REQUIRE(tiles * ((ff + kMoeBN - 1) / kMoeBN) < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_gate_up: launch too large");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == NV_DTYPE_BF16)
-        launch_grouped<__bf16, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
+        launch_grouped<__bf16, 1>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
                                      alpha, up_shift, (int)tiles, tile_rows, s);
     else
-        launch_grouped<float, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
+        launch_grouped<float, 1>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
                                     alpha, up_shift, (int)tiles, tile_rows, s);
     return check_launch("nv_moe_gate_up");
 }
@@ -336,10 +403,48 @@ extern "C" int nv_moe_down(const void* y, const void* down, const int32_t* sorte
     NV_REQUIRE(tiles * ((width + kMoeBN - 1) / kMoeBN) < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_down: launch too large");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == NV_DTYPE_BF16)
-        launch_grouped<__bf16, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f, 0.f,
+        launch_grouped<__bf16, 0>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f, 0.f,
                                       (int)tiles, tile_rows, s);
     else
-        launch_grouped<float, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f, 0.f,
+        launch_grouped<float, 0>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f, 0.f,
                                      (int)tiles, tile_rows, s);
     return check_launch("nv_moe_down");
+}
+
+extern "C" int nv_moe_route_grouped(const float* logits, const float* correction, int32_t* ids, float* weights, int64_t T,
+                                    int E, int top, int n_groups, int keep_groups, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(T >= 0 && E > 0 && E <= kMoeGroupedMaxE && top >= 1, NV_ERR_INVALID_ARG,
+               "nv_moe_route_grouped: E=%d must lie in 1 .. %d", E, kMoeGroupedMaxE);
+    NV_REQUIRE(n_groups >= 1 && E % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups, NV_ERR_INVALID_ARG,
+               "nv_moe_route_grouped: %d groups must divide E=%d and hold the %d kept", n_groups, E, keep_groups);
+    NV_REQUIRE(top <= keep_groups * (E / n_groups), NV_ERR_INVALID_ARG,
+               "nv_moe_route_grouped: top=%d exceeds the %d experts of the kept groups", top, keep_groups * (E / n_groups));
+    if (T == 0) return NV_OK;
+    NV_REQUIRE(logits && ids && weights, NV_ERR_INVALID_ARG, "nv_moe_route_grouped: null pointer");
+    NV_REQUIRE(T < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_route_grouped: launch too large");
+    hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream, logits, correction, ids,
+                       weights, E, top, n_groups, keep_groups);
+    return check_launch("nv_moe_route_grouped");
+}
+
+extern "C" int nv_moe_up_relu2(const void* h, int64_t h_stride, const void* up, const int32_t* sorted_pairs,
+                               const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width, int ff,
+                               int tile_rows, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(pairs >= 0 && E > 0 && top > 0 && width > 0 && ff > 0 && (tile_rows == 16 || tile_rows == 64),
+               NV_ERR_INVALID_ARG, "nv_moe_up_relu2: bad sizes");
+    if (pairs == 0) return NV_OK;
+    NV_REQUIRE(h && up && sorted_pairs && meta && y, NV_ERR_INVALID_ARG, "nv_moe_up_relu2: null pointer");
+    NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_moe_up_relu2: bad dtype");
+    const int64_t tiles = nv_moe_max_tiles(pairs, E, tile_rows);
+    NV_REQUIRE(tiles * ((ff + kMoeBN - 1) / kMoeBN) < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_up_relu2: launch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NV_DTYPE_BF16)
+        launch_grouped<__bf16, 2>(h, h_stride, up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, 0.f, 0.f, 0.f,
+                                  (int)tiles, tile_rows, s);
+    else
+        launch_grouped<float, 2>(h, h_stride, up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, 0.f, 0.f, 0.f,
+                                 (int)tiles, tile_rows, s);
+    return check_launch("nv_moe_up_relu2");
 }

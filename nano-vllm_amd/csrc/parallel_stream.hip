@@ -72,6 +72,10 @@ __global__ __launch_bounds__(kPsThreads) void hashed_bigram_embed_kernel(
         row[c] = v;
         ss += v * v;
     }
+    if (norm_w == nullptr) {                                   // no norm: a thread reads back its own columns
+        for (int c = tid; c < cols; c += kPsThreads) x[(int64_t)t * cols + c] = row[c];
+        return;
+    }
     ss = ps_block_sum(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)cols + eps);
     for (int c = tid; c < cols; c += kPsThreads) x[(int64_t)t * cols + c] = row[c] * rstd * norm_w[c];
@@ -159,7 +163,7 @@ extern "C" int nv_hashed_bigram_embed(const int64_t* ids, const int64_t* positio
     using namespace nv;
     NV_REQUIRE(T >= 0 && num_seqs >= 0 && cols > 0 && cols <= 16384, NV_ERR_INVALID_ARG, "nv_hashed_bigram_embed: bad sizes");
     if (T == 0 || num_seqs == 0) return NV_OK;
-    NV_REQUIRE(ids && positions && embed && norm_w && x && cu_seqlens_q, NV_ERR_INVALID_ARG,
+    NV_REQUIRE(ids && positions && embed && x && cu_seqlens_q, NV_ERR_INVALID_ARG,
                "nv_hashed_bigram_embed: null pointer");
     NV_REQUIRE(!bigram || (buckets > 0 && prev_state && state_slots), NV_ERR_INVALID_ARG,
                "nv_hashed_bigram_embed: a bigram table needs its bucket count and the carried ids");

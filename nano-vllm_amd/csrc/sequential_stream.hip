@@ -1,0 +1,215 @@
+// An fp32 residual stream whose sublayers run one after the other (pre-norm), each output scaled per column on its way
+// in, and what stands around its attention and feed-forward sublayers.
+//
+// nv_stream_boundary_scaled  per row, in place on the fp32 stream r:
+//                                r <- r + ls * (a1 + sigmoid(g) a2 + sum_j p_j)    (a1, a2 in the matmul dtype, g one raw
+//                                                                                  gate per row for a2, p_j fp32 parts such
+//                                                                                  as the weighted outputs of the chosen
+//                                                                                  experts, ls a scale per column; each
+//                                                                                  may be absent)
+//                                y32 / y <- r / sqrt(mean(r^2) + eps) * w          (fp32 and / or the matmul dtype; may
+//                                                                                  be absent)
+//                            so the stream is read and written once per sublayer.
+// nv_poly_norm               y = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e per row, powers element by element,
+//                            rms(u) = sqrt(mean(u^2) + eps) over the row, everything in fp32.
+// nv_head_norm_rope_store    in front of nv_attn_scoremod_paged when queries and keys are RMS-normed per head (one weight
+//                            [D] for all heads) and then rotated on their first rot_dims dimensions (pair (i, i + rot_dims/2)
+//                            by position * freq[i]): writes the prepared queries, scatters the prepared keys into the key
+//                            cache and the UNPREPARED keys into the value cache (this attention reads its values from the
+//                            keys as they come in).
+#include "nv_common.h"
+#include "../../include/nanovllm_hip_mixers.h"
+
+namespace nv {
+
+constexpr int kSsThreads = 256;
+
+__device__ __forceinline__ float ss_block_sum(float x, float* red) {
+    x = wave_sum(x);
+    const int w = threadIdx.x >> 6;
+    __syncthreads();                       // red may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) red[w] = x;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < kSsThreads / 64; ++i) t += red[i];
+    return t;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSsThreads) void stream_boundary_scaled_kernel(
+    float* __restrict__ resid, const T* __restrict__ add1, int64_t add1_stride, const T* __restrict__ add2,
+    int64_t add2_stride, const T* __restrict__ gate2, int64_t gate2_stride, const float* __restrict__ parts, int n_parts,
+    const float* __restrict__ col_scale, const float* __restrict__ norm_w, float eps, float* __restrict__ y32,
+    T* __restrict__ y, int cols) {
+    extern __shared__ float row[];
+    __shared__ float red[kSsThreads / 64];
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x;
+    float* rrow = resid + r * cols;
+    const float g2 = (add2 != nullptr && gate2 != nullptr) ? 1.0f / (1.0f + expf(-(float)gate2[r * gate2_stride])) : 1.0f;
+    float ss = 0.f;
+    for (int c = tid; c < cols; c += kSsThreads) {
+        float s = 0.f;
+        if (add1 != nullptr) s += (float)add1[r * add1_stride + c];
+        if (add2 != nullptr) s += g2 * (float)add2[r * add2_stride + c];
+        for (int j = 0; j < n_parts; ++j) s += parts[(r * n_parts + j) * cols + c];
+        if (col_scale != nullptr) s *= col_scale[c];
+        const float v = rrow[c] + s;
+        if (add1 != nullptr || add2 != nullptr || n_parts > 0) rrow[c] = v;
+        row[c] = v;
+        ss += v * v;
+    }
+    if (norm_w == nullptr) return;
+    const float rstd = 1.0f / sqrtf(ss_block_sum(ss, red) / (float)cols + eps);
+    for (int c = tid; c < cols; c += kSsThreads) {         // a thread reads back its own columns only
+        const float u = row[c] * rstd * norm_w[c];
+        if (y32 != nullptr) y32[r * cols + c] = u;
+        if (y != nullptr) y[r * cols + c] = (T)u;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSsThreads) void poly_norm_kernel(const T* __restrict__ x, int64_t x_stride,
+                                                               const float* __restrict__ coef, float eps,
+                                                               T* __restrict__ y, int cols) {
+    __shared__ float red[kSsThreads / 64];
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x;
+    const T* xr = x + r * x_stride;
+    float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+    for (int c = tid; c < cols; c += kSsThreads) {
+        const float z = (float)xr[c], z2 = z * z;
+        s2 += z2;
+        s4 += z2 * z2;
+        s6 += z2 * z2 * z2;
+    }
+    const float n = (float)cols;
+    const float r1 = coef[0] / sqrtf(ss_block_sum(s2, red) / n + eps);
+    const float r2 = coef[1] / sqrtf(ss_block_sum(s4, red) / n + eps);
+    const float r3 = coef[2] / sqrtf(ss_block_sum(s6, red) / n + eps);
+    const float shift = coef[3];
+    for (int c = tid; c < cols; c += kSsThreads) {
+        const float z = (float)xr[c], z2 = z * z;
+        y[r * cols + c] = (T)(r1 * z + r2 * z2 + r3 * (z2 * z) + shift);
+    }
+}
+
+// One wave per (token, head); heads 0 .. H-1 are the query's, H .. H+G-1 the key's.  A lane holds both halves of its
+// rotary pairs, so the rotation needs no exchange; the head is read twice (sum of squares, then output), the second
+// time from cache.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_rope_store_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, int64_t q_stride, int64_t k_stride, const float* __restrict__ q_norm,
+    const float* __restrict__ k_norm, float eps, const float* __restrict__ freq, int rot_dims,
+    const int64_t* __restrict__ positions, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int64_t items, int H, int G, int D) {
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= items) return;                         // (whole waves leave together)
+    const int lane = threadIdx.x & 63;
+    const int64_t t = item / (H + G);
+    const int head = (int)(item - t * (H + G));
+    const bool is_q = head < H;
+    const T* src = is_q ? q + t * q_stride + (int64_t)head * D : k + t * k_stride + (int64_t)(head - H) * D;
+    const float* w = is_q ? q_norm : k_norm;
+    T* dst;
+    T* raw = nullptr;
+    if (is_q) {
+        dst = q_out + (t * H + head) * D;
+    } else {
+        const int slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
+        if (slot < 0) return;
+        dst = k_cache + ((int64_t)slot * G + (head - H)) * D;
+        raw = v_cache + ((int64_t)slot * G + (head - H)) * D;
+    }
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) {
+        const float x = (float)src[d];
+        ss += x * x;
+        if (raw != nullptr) raw[d] = src[d];
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+    const int half = rot_dims >> 1;
+    const float p = (float)positions[t];
+    for (int i = lane; i < half; i += 64) {
+        const float u = (float)src[i] * rstd * w[i], v = (float)src[i + half] * rstd * w[i + half];
+        const float ang = p * freq[i];
+        const float c = cosf(ang), s = sinf(ang);
+        dst[i] = (T)(u * c - v * s);
+        dst[i + half] = (T)(v * c + u * s);
+    }
+    for (int d = rot_dims + lane; d < D; d += 64) dst[d] = (T)((float)src[d] * rstd * w[d]);
+}
+
+}  // namespace nv
+
+extern "C" int nv_stream_boundary_scaled(void* resid, const void* add1, int64_t add1_stride, const void* add2,
+                                         int64_t add2_stride, const void* gate2, int64_t gate2_stride, const float* parts,
+                                         int n_parts, const float* col_scale, const float* norm_w, float eps, float* y32,
+                                         void* y, int dtype, int64_t rows, int cols, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(rows >= 0 && cols > 0 && cols <= 16384, NV_ERR_INVALID_ARG, "nv_stream_boundary_scaled: bad sizes");
+    if (rows == 0) return NV_OK;
+    NV_REQUIRE(resid, NV_ERR_INVALID_ARG, "nv_stream_boundary_scaled: null stream");
+    NV_REQUIRE(!parts || n_parts > 0, NV_ERR_INVALID_ARG, "nv_stream_boundary_scaled: parts without a count");
+    NV_REQUIRE(!gate2 || add2, NV_ERR_INVALID_ARG, "nv_stream_boundary_scaled: a gate without its input");
+    NV_REQUIRE(!norm_w || y32 || y, NV_ERR_INVALID_ARG, "nv_stream_boundary_scaled: the norm needs an output");
+    NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_stream_boundary_scaled: bad dtype");
+    NV_REQUIRE(rows < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_stream_boundary_scaled: launch too large");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t smem = sizeof(float) * (size_t)cols;
+    const int np = parts ? n_parts : 0;
+    if (dtype == NV_DTYPE_BF16)
+        hipLaunchKernelGGL(stream_boundary_scaled_kernel<__bf16>, dim3((unsigned)rows), dim3(kSsThreads), smem, s,
+                           (float*)resid, (const __bf16*)add1, add1_stride, (const __bf16*)add2, add2_stride,
+                           (const __bf16*)gate2, gate2_stride, parts, np, col_scale, norm_w, eps, y32, (__bf16*)y, cols);
+    else
+        hipLaunchKernelGGL(stream_boundary_scaled_kernel<float>, dim3((unsigned)rows), dim3(kSsThreads), smem, s,
+                           (float*)resid, (const float*)add1, add1_stride, (const float*)add2, add2_stride,
+                           (const float*)gate2, gate2_stride, parts, np, col_scale, norm_w, eps, y32, (float*)y, cols);
+    return check_launch("nv_stream_boundary_scaled");
+}
+
+extern "C" int nv_poly_norm(const void* x, int64_t x_stride, const float* coef, float eps, void* y, int dtype, int64_t rows,
+                            int cols, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(rows >= 0 && cols > 0 && x_stride >= cols, NV_ERR_INVALID_ARG, "nv_poly_norm: bad sizes");
+    if (rows == 0) return NV_OK;
+    NV_REQUIRE(x && coef && y, NV_ERR_INVALID_ARG, "nv_poly_norm: null pointer");
+    NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_poly_norm: bad dtype");
+    NV_REQUIRE(rows < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_poly_norm: launch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NV_DTYPE_BF16)
+        hipLaunchKernelGGL(poly_norm_kernel<__bf16>, dim3((unsigned)rows), dim3(kSsThreads), 0, s, (const __bf16*)x, x_stride,
+                           coef, eps, (__bf16*)y, cols);
+    else
+        hipLaunchKernelGGL(poly_norm_kernel<float>, dim3((unsigned)rows), dim3(kSsThreads), 0, s, (const float*)x, x_stride,
+                           coef, eps, (float*)y, cols);
+    return check_launch("nv_poly_norm");
+}
+
+extern "C" int nv_head_norm_rope_store(const void* q, const void* k, int64_t q_stride, int64_t k_stride, const float* q_norm,
+                                       const float* k_norm, float eps, const float* freq, int rot_dims,
+                                       const int64_t* positions, const int32_t* slot_mapping, void* q_out, void* k_cache,
+                                       void* v_cache, int dtype, int64_t T, int H, int G, int D, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(T >= 0 && H > 0 && G > 0 && D > 0, NV_ERR_INVALID_ARG, "nv_head_norm_rope_store: bad sizes");
+    NV_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= D, NV_ERR_INVALID_ARG,
+               "nv_head_norm_rope_store: rot_dims=%d must be even and at most D=%d", rot_dims, D);
+    if (T == 0) return NV_OK;
+    NV_REQUIRE(q && k && q_norm && k_norm && positions && q_out && k_cache && v_cache && (freq || rot_dims == 0),
+               NV_ERR_INVALID_ARG, "nv_head_norm_rope_store: null pointer");
+    NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_head_norm_rope_store: bad dtype");
+    const int64_t items = T * (H + G), grid = (items + 3) / 4;
+    NV_REQUIRE(grid < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_head_norm_rope_store: launch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NV_DTYPE_BF16)
+        hipLaunchKernelGGL(head_norm_rope_store_kernel<__bf16>, dim3((unsigned)grid), dim3(256), 0, s, (const __bf16*)q,
+                           (const __bf16*)k, q_stride, k_stride, q_norm, k_norm, eps, freq, rot_dims, positions, slot_mapping,
+                           (__bf16*)q_out, (__bf16*)k_cache, (__bf16*)v_cache, items, H, G, D);
+    else
+        hipLaunchKernelGGL(head_norm_rope_store_kernel<float>, dim3((unsigned)grid), dim3(256), 0, s, (const float*)q,
+                           (const float*)k, q_stride, k_stride, q_norm, k_norm, eps, freq, rot_dims, positions, slot_mapping,
+                           (float*)q_out, (float*)k_cache, (float*)v_cache, items, H, G, D);
+    return check_launch("nv_head_norm_rope_store");
+}

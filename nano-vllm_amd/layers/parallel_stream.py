@@ -21,13 +21,14 @@ stream_boundary_pair = ops.stream_boundary_pair
 
 class HashedBigramEmbedding(nn.Module):
     def __init__(self, vocab: int, width: int, buckets: int, mul_prev: int, mul_cur: int, eps: float, dtype=None,
-                 device=None):
-        """buckets = 0: no bigram table (the embedding row alone is normed)."""
+                 device=None, normed: bool = True):
+        """buckets = 0: no bigram table (the embedding row alone is normed).  normed=False: the sum of the rows goes
+        into the stream as it is."""
         super().__init__()
         self.buckets, self.mul_prev, self.mul_cur, self.eps = int(buckets), int(mul_prev), int(mul_cur), float(eps)
         self.weight = nn.Parameter(torch.zeros(vocab, width, dtype=dtype, device=device))
         self.bigram = nn.Parameter(torch.zeros(buckets + 1, width, dtype=dtype, device=device)) if buckets else None
-        self.norm = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device))
+        self.norm = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device)) if normed else None
 
     def forward(self, ids: torch.Tensor, positions: torch.Tensor, prev_state: torch.Tensor | None) -> torch.Tensor:
         """ids, positions [T] int64; prev_state [slots] int64; returns the stream [T, W] float32."""

@@ -109,9 +109,20 @@ def _divadra_model(cfg, dtype=torch.bfloat16, device="cuda", **kw):
     return DivadraForCausalLM(cfg, dtype=dtype, device=device, **kw)
 
 
+def _tutedra_config(raw: dict):
+    from .tutedra import TutedraConfig
+    return TutedraConfig.from_dict(raw)
+
+
+def _tutedra_model(cfg, dtype=torch.bfloat16, device="cuda", **kw):
+    from .tutedra import TutedraForCausalLM
+    return TutedraForCausalLM(cfg, dtype=dtype, device=device, **kw)
+
+
 register(["Qwen3ForCausalLM", "Qwen3"], _qwen3_config, lambda cfg, **kw: _qwen3_model(cfg, **kw))
 register(["LlamaForCausalLM", "Llama"], lambda raw: _qwen3_config({**raw, "qk_norm": False}),
          lambda cfg, **kw: _qwen3_model(cfg, **kw))
 register(["Buvalix", "BuvalixForCausalLM"], _buvalix_config, _buvalix_model)
 register(["Benarax", "BenaraxForCausalLM"], _benarax_config, _benarax_model)
 register(["Divadra", "DivadraForCausalLM"], _divadra_config, _divadra_model)
+register(["Tutedra", "TutedraForCausalLM"], _tutedra_config, _tutedra_model)

@@ -801,11 +801,12 @@ def _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots):
 
 
 def hashed_bigram_embed(ids: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, bigram: Optional[torch.Tensor],
-                        mul_prev: int, mul_cur: int, norm_weight: torch.Tensor, eps: float,
+                        mul_prev: int, mul_cur: int, norm_weight: Optional[torch.Tensor], eps: float,
                         prev_state: Optional[torch.Tensor], cu_seqlens_q: torch.Tensor,
                         state_slots: Optional[torch.Tensor]) -> torch.Tensor:
-    """x = rmsnorm(embed[id] + bigram[hash(previous id, id)]) * norm_weight as a float32 stream [T, W]; the last row
-    of the bigram table serves position 0; prev_state [slots] int64 carries each sequence's last id."""
+    """x = rmsnorm(embed[id] + bigram[hash(previous id, id)]) * norm_weight as a float32 stream [T, W] (norm_weight None:
+    the sum as it is); the last row of the bigram table serves position 0; prev_state [slots] int64 carries each
+    sequence's last id."""
     dt = _dt(embed, "embed")
     T, W = ids.numel(), embed.shape[1]
     for t, n in ((ids, "ids"), (positions, "positions")):
@@ -826,7 +827,7 @@ def hashed_bigram_embed(ids: torch.Tensor, positions: torch.Tensor, embed: torch
     x = torch.empty((T, W), dtype=torch.float32, device=embed.device)
     dll = _lib.mixers()
     rc = dll.nv_hashed_bigram_embed(ids.data_ptr(), positions.data_ptr(), embed.data_ptr(), _ptr(bigram), buckets,
-                                    int(mul_prev), int(mul_cur), _f32c(norm_weight, "norm_weight"), float(eps),
+                                    int(mul_prev), int(mul_cur), _f32c(norm_weight, "norm_weight") or None, float(eps),
                                     _ptr(prev_state) if bigram is not None else None, x.data_ptr(),
                                     cu_seqlens_q.data_ptr(), _ptr(state_slots) if bigram is not None else None, B, T, W,
                                     dt, _stream(embed))
@@ -1127,5 +1128,237 @@ def moe_table_experts(h: torch.Tensor, ids: torch.Tensor, gate_up: torch.Tensor,
                                       meta.data_ptr(), y.data_ptr(), dt, P, E, int(top), W, ff, float("inf"), 1.0, 0.0,
                                       rows, s), "nv_moe_gate_up_act", dll)
     _lib.check(dll.nv_moe_down(y.data_ptr(), down.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), wgt.data_ptr(),
+                               out.data_ptr(), dt, P, E, W, ff, rows, s), "nv_moe_down", dll)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Pre-norm fp32 stream with per-column output scales, memories written before they are read (exponential-gate matrix
+# memory, gated-write recurrence), attention whose values are its un-normed keys, polynomial-of-norms activation,
+# sigmoid routing over groups of squared-ReLU experts.
+# ---------------------------------------------------------------------------------------------------------
+def stream_boundary_scaled(x: torch.Tensor, add: Optional[torch.Tensor] = None, gated: Optional[tuple] = None,
+                           parts: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None,
+                           norm: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                           out_dtype: Optional[torch.dtype] = None, want_f32: bool = False):
+    """One sublayer boundary of a pre-norm fp32 stream x [T, W], in place:
+    x += col_scale * (add + sigmoid(g) * a2 + parts.sum(1)) with gated = (a2 [T, W], g [T] raw gate, one per row);
+    norm: the RMS-norm weight of the updated stream AS APPLIED (a one-plus weight is folded by the caller).
+    Returns (h32, h): the norm in float32 (if want_f32) and in out_dtype (if given); None for each part not asked for."""
+    _need(x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(),
+          "the stream must be a contiguous float32 [tokens, width] GPU tensor")
+    rows, cols = x.shape
+    a2, g2 = gated if gated is not None else (None, None)
+    ins = [t for t in (add, a2) if t is not None]
+    dt_t = out_dtype or (ins[0].dtype if ins else torch.float32)
+    _need(dt_t in (_BF16, torch.float32), "the matmul dtype must be bfloat16 or float32")
+    dt = _lib.DTYPE_BF16 if dt_t == _BF16 else _lib.DTYPE_F32
+    for t in ins:
+        _rows2d(t, "input")
+        _need(t.shape == x.shape and t.dtype == dt_t and t.is_cuda, "inputs must match the stream's shape, in the matmul dtype")
+    if g2 is not None:
+        _need(g2.is_cuda and g2.dtype == dt_t and g2.dim() == 1 and g2.numel() == rows, "the gate must be [T] of the matmul dtype")
+    n_parts = 0
+    if parts is not None:
+        _need(parts.is_cuda and parts.dtype == torch.float32 and parts.is_contiguous() and parts.dim() == 3
+              and parts.shape[0] == rows and parts.shape[2] == cols, "parts must be contiguous float32 [T, n, W]")
+        n_parts = parts.shape[1]
+    for w in (col_scale, norm):
+        _need(w is None or w.numel() == cols, "column scale and norm weight must be [width]")
+    y32 = y = None
+    if norm is not None:
+        if want_f32:
+            y32 = torch.empty((rows, cols), dtype=torch.float32, device=x.device)
+        if out_dtype is not None:
+            y = torch.empty((rows, cols), dtype=out_dtype, device=x.device)
+        _need(y32 is not None or y is not None, "the norm needs an output")
+    dll = _lib.mixers()
+    rc = dll.nv_stream_boundary_scaled(x.data_ptr(), _ptr(add), add.stride(0) if add is not None else 0, _ptr(a2),
+                                       a2.stride(0) if a2 is not None else 0, _ptr(g2), g2.stride(0) if g2 is not None else 0,
+                                       _ptr(parts) if n_parts else None, n_parts, _f32c(col_scale, "col_scale") or None,
+                                       _f32c(norm, "norm") or None, float(eps), _ptr(y32), _ptr(y), dt, rows, cols,
+                                       _stream(x))
+    _lib.check(rc, "nv_stream_boundary_scaled", dll)
+    return y32, y
+
+
+def poly_norm(x: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """coef[0] x / rms(x) + coef[1] x^2 / rms(x^2) + coef[2] x^3 / rms(x^3) + coef[3] per row of x [T, C]; coef: 4 float32
+    on the device."""
+    dt = _dt(x, "x")
+    _rows2d(x, "x")
+    _need(coef.numel() == 4, "coef must hold four numbers")
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    _lib.check(dll.nv_poly_norm(x.data_ptr(), x.stride(0), _f32c(coef, "coef"), float(eps), y.data_ptr(), dt, x.shape[0],
+                                x.shape[1], _stream(x)), "nv_poly_norm", dll)
+    return y
+
+
+def causal_conv(x: torch.Tensor, weight: torch.Tensor, conv_state: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                silu: bool = False) -> torch.Tensor:
+    """Causal conv over time per channel of x [T, C] (+ bias, then SiLU if asked); weight [C, taps] float32; conv_state
+    [num_slots, taps - 1, C] (x's dtype) carries each sequence's last inputs and is updated."""
+    dt = _dt(x, "x")
+    _rows2d(x, "x")
+    T, Cc = x.shape
+    taps = weight.shape[1]
+    _need(weight.shape[0] == Cc and (bias is None or bias.numel() == Cc), "weight must be [channels, taps], bias [channels]")
+    _need(conv_state.is_cuda and conv_state.dtype == x.dtype and conv_state.is_contiguous()
+          and conv_state.shape[1:] == (taps - 1, Cc), "conv_state must be contiguous [slots, taps - 1, C] of x's dtype")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    y = torch.empty((T, Cc), dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_causal_conv_act(x.data_ptr(), x.stride(0), _f32c(weight, "weight"), _f32c(bias, "bias") or None,
+                                conv_state.data_ptr(), y.data_ptr(), y.stride(0), cu_seqlens_q.data_ptr(),
+                                cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, T, Cc, taps, 1 if silu else 0, dt,
+                                _stream(x))
+    _lib.check(rc, "nv_causal_conv_act", dll)
+    return y
+
+
+def head_norm_rope_store(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, q_norm: torch.Tensor,
+                         k_norm: torch.Tensor, eps: float, freq: Optional[torch.Tensor], rot_dims: int,
+                         slot_mapping: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+    """Per-head RMS norm of q [T, H, D] and k [T, G, D] (weights [D]), rotate-half rotary on the first rot_dims
+    dimensions, scatter of the prepared k into k_cache and of k as given into v_cache; returns the prepared q."""
+    dt = _dt(q, "q")
+    for t, n in ((q, "q"), (k, "k")):
+        _rows_ok(t, n)
+        _need(t.dtype == q.dtype, "q, k must have one dtype")
+    T, H, D = q.shape
+    G = k.shape[1]
+    _need(k.shape == (T, G, D), "k rows do not match q")
+    _need(positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T,
+          "positions must be a contiguous int64 [tokens] GPU tensor")
+    _need(q_norm.numel() == D and k_norm.numel() == D, "norm weights must be [D]")
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "slot_mapping length != number of tokens")
+    for c in (k_cache, v_cache):
+        _need(c.is_cuda and c.is_contiguous() and c.dtype == q.dtype and c.dim() == 4 and c.shape[2:] == (G, D),
+              "caches must be contiguous [num_blocks, block_size, G, D] of q's dtype")
+    if rot_dims:
+        _need(freq is not None and freq.numel() == rot_dims // 2, "freq must hold rot_dims / 2 frequencies")
+    q_out = torch.empty((T, H, D), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_head_norm_rope_store(q.data_ptr(), k.data_ptr(), q.stride(0), k.stride(0), _f32c(q_norm, "q_norm"),
+                                     _f32c(k_norm, "k_norm"), float(eps), _f32c(freq, "freq") or None, int(rot_dims),
+                                     positions.data_ptr(), _ptr(slot_mapping), q_out.data_ptr(), k_cache.data_ptr(),
+                                     v_cache.data_ptr(), dt, T, H, G, D, _stream(q))
+    _lib.check(rc, "nv_head_norm_rope_store", dll)
+    return q_out
+
+
+def mlstm_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates_pre: torch.Tensor, gate_raw: torch.Tensor,
+                 i_bias: torch.Tensor, f_bias: torch.Tensor, norm_weight: torch.Tensor, state: torch.Tensor,
+                 norm_state: torch.Tensor, max_state: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
+                 state_slots: torch.Tensor, eps: float, gate_cap: float, q_scale: float) -> torch.Tensor:
+    """Matrix memory with exponential gates over a step's rows; q, k: [T, H, Dk]; v: [T, H, Dv]; gates_pre [T, 2 H] float32
+    (input-gate columns, then forget-gate columns, without bias); gate_raw [T, H * Dv]; state [slots, H, Dk, Dv],
+    norm_state [slots, H, Dk], max_state [slots, H] float32, updated in place; returns [T, H * Dv]."""
+    dt = _dt(q, "q")
+    T, H, Dk = q.shape
+    Dv = v.shape[2]
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _rows_ok(t, n)
+        _need(t.dtype == q.dtype, "q, k, v must have one dtype")
+    _need(k.shape == (T, H, Dk) and v.shape[:2] == (T, H), "q / k / v rows differ")
+    _rows2d(gate_raw, "gate_raw")
+    _need(gate_raw.shape == (T, H * Dv) and gate_raw.dtype == q.dtype, "gate_raw must be [T, H * Dv] of q's dtype")
+    _need(gates_pre.is_cuda and gates_pre.dtype == torch.float32 and gates_pre.dim() == 2 and gates_pre.stride(1) == 1
+          and gates_pre.shape == (T, 2 * H), "gates_pre must be float32 [T, 2 H]")
+    for t, n, shape in ((state, "state", (H, Dk, Dv)), (norm_state, "norm_state", (H, Dk)), (max_state, "max_state", (H,))):
+        _need(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.shape[1:] == shape,
+              f"{n} must be contiguous float32 [slots, {shape}]")
+    _need(i_bias.numel() == H and f_bias.numel() == H and norm_weight.numel() == H * Dv, "constant shapes")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_mlstm_memory(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0),
+                             gates_pre.data_ptr(), gates_pre.data_ptr() + 4 * H, gates_pre.stride(0), gate_raw.data_ptr(),
+                             gate_raw.stride(0), _f32c(i_bias, "i_bias"), _f32c(f_bias, "f_bias"),
+                             _f32c(norm_weight, "norm_weight"), state.data_ptr(), norm_state.data_ptr(),
+                             max_state.data_ptr(), out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(),
+                             cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, H, Dk, Dv, float(eps), float(gate_cap),
+                             float(q_scale), dt, _stream(q))
+    _lib.check(rc, "nv_mlstm_memory", dll)
+    return out
+
+
+def gated_write_memory(q: torch.Tensor, f_raw: torch.Tensor, v: torch.Tensor, f_bias: torch.Tensor, lower: torch.Tensor,
+                       norm_weight: torch.Tensor, state: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                       cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor, eps: float) -> torch.Tensor:
+    """Gated linear recurrence whose forget gate decides what is written; q, f_raw: [T, H, Dk] as projected; v: [T, H, Dv];
+    f_bias, lower [H * Dk], norm_weight [Dv] float32; state [slots, H, Dk, Dv] float32 updated in place; returns
+    [T, H * Dv]."""
+    dt = _dt(q, "q")
+    T, H, Dk = q.shape
+    Dv = v.shape[2]
+    for t, n in ((q, "q"), (f_raw, "f_raw"), (v, "v")):
+        _rows_ok(t, n)
+        _need(t.dtype == q.dtype, "q, f_raw, v must have one dtype")
+    _need(f_raw.shape == (T, H, Dk) and v.shape[:2] == (T, H), "q / f_raw / v rows differ")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, Dk, Dv),
+          "state must be contiguous float32 [slots, H, Dk, Dv]")
+    _need(f_bias.numel() == H * Dk and lower.numel() == H * Dk and norm_weight.numel() == Dv, "constant shapes")
+    B = _seq_meta(cu_seqlens_q, cu_seqlens_k, state_slots)
+    out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_gated_write_memory(q.data_ptr(), f_raw.data_ptr(), v.data_ptr(), q.stride(0), f_raw.stride(0), v.stride(0),
+                                   _f32c(f_bias, "f_bias"), _f32c(lower, "lower"), _f32c(norm_weight, "norm_weight"),
+                                   state.data_ptr(), out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(),
+                                   cu_seqlens_k.data_ptr(), state_slots.data_ptr(), B, H, Dk, Dv, float(eps), dt, _stream(q))
+    _lib.check(rc, "nv_gated_write_memory", dll)
+    return out
+
+
+def moe_route_grouped(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_groups: int,
+                      keep_groups: int) -> tuple:
+    """(ids [T, top] int32, weights [T, top] float32): sigmoid scores, choice on score + correction within the best
+    groups, weights the plain scores of the chosen."""
+    _need(logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and logits.dim() == 2,
+          "logits must be contiguous float32 [T, E]")
+    T, E = logits.shape
+    _need(correction is None or correction.numel() == E, "correction must be [E]")
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    wgt = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    dll = _lib.mixers()
+    _lib.check(dll.nv_moe_route_grouped(logits.data_ptr(), _f32c(correction, "correction") or None, ids.data_ptr(),
+                                        wgt.data_ptr(), T, E, int(top), int(n_groups), int(keep_groups), _stream(logits)),
+               "nv_moe_route_grouped", dll)
+    return ids, wgt
+
+
+def moe_relu2_experts(h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, up: torch.Tensor,
+                      down: torch.Tensor) -> torch.Tensor:
+    """Squared-ReLU experts for given choices: h [T, W]; ids [T, top] int32; weights [T, top] float32; up [E, ff, W];
+    down [E, W, ff].  Returns the weighted outputs [T, top, W] float32 (the stream update sums them)."""
+    dt = _dt(h, "h")
+    _rows2d(h, "h")
+    T, W = h.shape
+    E, ff = up.shape[0], up.shape[1]
+    top = ids.shape[1]
+    _need(ids.is_cuda and ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape == (T, top)
+          and weights.is_cuda and weights.dtype == torch.float32 and weights.is_contiguous() and weights.shape == (T, top),
+          "ids must be contiguous int32 [T, top], weights float32 [T, top]")
+    _need(up.is_cuda and down.is_cuda and up.is_contiguous() and down.is_contiguous() and up.dtype == h.dtype
+          and down.dtype == h.dtype and up.shape == (E, ff, W) and down.shape == (E, W, ff),
+          "up must be [E, ff, W] and down [E, W, ff], contiguous, of h's dtype")
+    dll = _lib.mixers()
+    dev, P, s = h.device, T * top, _stream(h)
+    out = torch.empty((T, top, W), dtype=torch.float32, device=dev)
+    if T == 0:
+        return out
+    rows = dll.nv_moe_tile_rows(P, E)
+    tiles = dll.nv_moe_max_tiles(P, E, rows)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    meta = torch.empty(1 + 3 * tiles, dtype=torch.int32, device=dev)
+    _lib.check(dll.nv_moe_align(ids.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), P, E, rows, s), "nv_moe_align", dll)
+    y = torch.empty((P, ff), dtype=h.dtype, device=dev)
+    _lib.check(dll.nv_moe_up_relu2(h.data_ptr(), h.stride(0), up.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(),
+                                   y.data_ptr(), dt, P, E, int(top), W, ff, rows, s), "nv_moe_up_relu2", dll)
+    _lib.check(dll.nv_moe_down(y.data_ptr(), down.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), weights.data_ptr(),
                                out.data_ptr(), dt, P, E, W, ff, rows, s), "nv_moe_down", dll)
     return out

@@ -24,12 +24,12 @@ def _spans(ctx):
 
 
 class HashedBigramEmbedding(nn.Module):
-    def __init__(self, vocab, width, buckets, mul_prev, mul_cur, eps, dtype=None, device=None):
+    def __init__(self, vocab, width, buckets, mul_prev, mul_cur, eps, dtype=None, device=None, normed=True):
         super().__init__()
         self.buckets, self.mul_prev, self.mul_cur, self.eps = int(buckets), int(mul_prev), int(mul_cur), float(eps)
         self.weight = nn.Parameter(torch.zeros(vocab, width, dtype=dtype, device=device))
         self.bigram = nn.Parameter(torch.zeros(buckets + 1, width, dtype=dtype, device=device)) if buckets else None
-        self.norm = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device))
+        self.norm = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device)) if normed else None
 
     def forward(self, ids, positions, prev_state):
         x = self.weight[ids].float()
@@ -42,7 +42,7 @@ class HashedBigramEmbedding(nn.Module):
                     rows[r0] = self.buckets
                 prev_state[slot] = ids[r0 + nq - 1]
             x = x + self.bigram[rows].float()
-        return _unit_rms(x, self.eps) * self.norm
+        return _unit_rms(x, self.eps) * self.norm if self.norm is not None else x
 
 
 def stream_boundary_pair(x, adds=(), parts=None, parts_scale=1.0, normed=(), normed_mult=1.0, norms=(), eps=1e-5,
