@@ -29,15 +29,28 @@ def bound(dtype):
     return 5e-5 if dtype == torch.float32 else 6e-2
 
 
+def per_position(got, want):
+    d = got.float() - want.float()
+    d = d - d.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / want.float().pow(2).mean().sqrt()
+
+
 def assert_close_to_oracle(got, cfg, ck, prompt, dtype, what=""):
+    """float32: every position.  bfloat16: against what the oracle's own bfloat16 evaluation loses per position; a fault
+    moves most positions, while rounding can turn a close call of a router (two experts whose scores differ by less
+    than the rounding) and move that position and the few behind it that read it through a state: at most one
+    position in ten may exceed three times the oracle's loss, and the median must not move."""
     want = oracle_logits(cfg, ck, prompt, torch.float32)
     assert got.shape == want.shape
-    err = rel_err(got, want)
     if dtype == torch.float32:
+        err = rel_err(got, want)
         assert err < bound(dtype), (what, err)
     else:
-        noise = rel_err(oracle_logits(cfg, ck, prompt, torch.bfloat16), want)
-        assert err < 3 * noise, (what, err, noise)
+        err = per_position(got, want)
+        noise = per_position(oracle_logits(cfg, ck, prompt, torch.bfloat16), want)
+        limit = 3 * torch.clamp(noise, min=noise.median().item()) + 1e-3
+        assert int((err > limit).sum()) <= max(1, err.numel() // 10), (what, (err / limit).topk(5).values.tolist())
+        assert err.median().item() <= 2 * noise.median().item() + 1e-3, (what, err.median().item(), noise.median().item())
 
 
 def tokens(n, seed, vocab=83):
