@@ -71,6 +71,9 @@ def parse():
     ap.add_argument("--divadra", action="store_true",
                     help="instead of the default workload: the Divadra kernels and model beside Benarax at equal sizes "
                          "(one GPU, random weights), one JSON line; switched off unless NV_ALLOW_DIVADRA_BENCH=1")
+    ap.add_argument("--tutedra", action="store_true",
+                    help="instead of the default workload: the Tutedra kernels and model beside Benarax at equal sizes "
+                         "(one GPU, random weights), one JSON line")
     return ap.parse_args()
 
 
@@ -802,6 +805,12 @@ def main():
             raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
         from tools.benarax_bench import run as benarax_run
         print(json.dumps(benarax_run("cuda:0")))
+        return
+    if args.tutedra:
+        if not torch.cuda.is_available():
+            raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
+        from tools.tutedra_bench import run as tutedra_run
+        print(json.dumps(tutedra_run("cuda:0")))
         return
     if args.divadra:
         if not torch.cuda.is_available():
