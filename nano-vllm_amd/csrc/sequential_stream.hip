@@ -69,29 +69,97 @@ __global__ __launch_bounds__(kSsThreads) void stream_boundary_scaled_kernel(
     }
 }
 
-template <typename T>
+// 16 bytes of a row as floats (8 bfloat16 or 4 float32).
+template <typename T> struct SsPiece;
+template <> struct SsPiece<__bf16> {
+    static constexpr int n = 8;
+    static __device__ __forceinline__ void load(const __bf16* p, float* o) {
+        const uint4 u = *(const uint4*)p;
+        o[0] = bf16_lo(u.x); o[1] = bf16_hi(u.x); o[2] = bf16_lo(u.y); o[3] = bf16_hi(u.y);
+        o[4] = bf16_lo(u.z); o[5] = bf16_hi(u.z); o[6] = bf16_lo(u.w); o[7] = bf16_hi(u.w);
+    }
+    static __device__ __forceinline__ void store(__bf16* p, const float* o) {
+        *(uint4*)p = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+    }
+};
+template <> struct SsPiece<float> {
+    static constexpr int n = 4;
+    static __device__ __forceinline__ void load(const float* p, float* o) {
+        const float4 u = *(const float4*)p;
+        o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float* o) { *(float4*)p = make_float4(o[0], o[1], o[2], o[3]); }
+};
+
+// The three sums of a row (z^2, z^4, z^6) are reduced together: one exchange through LDS.  VEC: the row is walked in
+// 16-byte pieces (the host checks size, stride and alignment); the second walk finds the row in cache.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kSsThreads) void poly_norm_kernel(const T* __restrict__ x, int64_t x_stride,
                                                                const float* __restrict__ coef, float eps,
                                                                T* __restrict__ y, int cols) {
-    __shared__ float red[kSsThreads / 64];
+    constexpr int N = SsPiece<T>::n;
+    __shared__ float red[3][kSsThreads / 64];
     const int64_t r = blockIdx.x;
     const int tid = threadIdx.x;
     const T* xr = x + r * x_stride;
     float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-    for (int c = tid; c < cols; c += kSsThreads) {
-        const float z = (float)xr[c], z2 = z * z;
-        s2 += z2;
-        s4 += z2 * z2;
-        s6 += z2 * z2 * z2;
+    if constexpr (VEC) {
+        for (int c = tid * N; c < cols; c += kSsThreads * N) {
+            float z[N];
+            SsPiece<T>::load(xr + c, z);
+#pragma unroll
+            for (int e = 0; e < N; ++e) {
+                const float z2 = z[e] * z[e];
+                s2 += z2;
+                s4 += z2 * z2;
+                s6 += z2 * z2 * z2;
+            }
+        }
+    } else {
+        for (int c = tid; c < cols; c += kSsThreads) {
+            const float z = (float)xr[c], z2 = z * z;
+            s2 += z2;
+            s4 += z2 * z2;
+            s6 += z2 * z2 * z2;
+        }
+    }
+    s2 = wave_sum(s2);
+    s4 = wave_sum(s4);
+    s6 = wave_sum(s6);
+    if ((tid & 63) == 0) {
+        red[0][tid >> 6] = s2;
+        red[1][tid >> 6] = s4;
+        red[2][tid >> 6] = s6;
+    }
+    __syncthreads();
+    s2 = s4 = s6 = 0.f;
+#pragma unroll
+    for (int i = 0; i < kSsThreads / 64; ++i) {
+        s2 += red[0][i];
+        s4 += red[1][i];
+        s6 += red[2][i];
     }
     const float n = (float)cols;
-    const float r1 = coef[0] / sqrtf(ss_block_sum(s2, red) / n + eps);
-    const float r2 = coef[1] / sqrtf(ss_block_sum(s4, red) / n + eps);
-    const float r3 = coef[2] / sqrtf(ss_block_sum(s6, red) / n + eps);
+    const float r1 = coef[0] / sqrtf(s2 / n + eps);
+    const float r2 = coef[1] / sqrtf(s4 / n + eps);
+    const float r3 = coef[2] / sqrtf(s6 / n + eps);
     const float shift = coef[3];
-    for (int c = tid; c < cols; c += kSsThreads) {
-        const float z = (float)xr[c], z2 = z * z;
-        y[r * cols + c] = (T)(r1 * z + r2 * z2 + r3 * (z2 * z) + shift);
+    if constexpr (VEC) {
+        for (int c = tid * N; c < cols; c += kSsThreads * N) {
+            float z[N];
+            SsPiece<T>::load(xr + c, z);
+#pragma unroll
+            for (int e = 0; e < N; ++e) {
+                const float z2 = z[e] * z[e];
+                z[e] = r1 * z[e] + r2 * z2 + r3 * (z2 * z[e]) + shift;
+            }
+            SsPiece<T>::store(y + r * cols + c, z);
+        }
+    } else {
+        for (int c = tid; c < cols; c += kSsThreads) {
+            const float z = (float)xr[c], z2 = z * z;
+            y[r * cols + c] = (T)(r1 * z + r2 * z2 + r3 * (z2 * z) + shift);
+        }
     }
 }
 
@@ -141,6 +209,87 @@ __global__ __launch_bounds__(256) void head_norm_rope_store_kernel(
     for (int d = rot_dims + lane; d < D; d += 64) dst[d] = (T)((float)src[d] * rstd * w[d]);
 }
 
+// The same for heads of at most 128 dimensions with even sizes: a lane keeps two neighbouring dimensions in registers (one
+// 4- or 8-byte load), the rotary partner (half the rotated part away) comes from another lane by a shuffle, so the head
+// is read once and nothing waits on a second trip to memory.
+template <typename T> struct SsPair;
+template <> struct SsPair<__bf16> {
+    static __device__ __forceinline__ void load(const __bf16* p, float& a, float& b) {
+        const uint32_t u = *(const uint32_t*)p;
+        a = bf16_lo(u);
+        b = bf16_hi(u);
+    }
+    static __device__ __forceinline__ void store(__bf16* p, float a, float b) { *(uint32_t*)p = pack_bf16(a, b); }
+    static __device__ __forceinline__ void copy(__bf16* d, const __bf16* s) { *(uint32_t*)d = *(const uint32_t*)s; }
+};
+template <> struct SsPair<float> {
+    static __device__ __forceinline__ void load(const float* p, float& a, float& b) {
+        const float2 u = *(const float2*)p;
+        a = u.x;
+        b = u.y;
+    }
+    static __device__ __forceinline__ void store(float* p, float a, float b) { *(float2*)p = make_float2(a, b); }
+    static __device__ __forceinline__ void copy(float* d, const float* s) { *(float2*)d = *(const float2*)s; }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_rope_store_pairs_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, int64_t q_stride, int64_t k_stride, const float* __restrict__ q_norm,
+    const float* __restrict__ k_norm, float eps, const float* __restrict__ freq, int rot_dims,
+    const int64_t* __restrict__ positions, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int64_t items, int H, int G, int D) {
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= items) return;                         // (whole waves leave together)
+    const int lane = threadIdx.x & 63;
+    const int64_t t = item / (H + G);
+    const int head = (int)(item - t * (H + G));
+    const bool is_q = head < H;
+    const T* src = is_q ? q + t * q_stride + (int64_t)head * D : k + t * k_stride + (int64_t)(head - H) * D;
+    const float* w = is_q ? q_norm : k_norm;
+    T* dst;
+    T* raw = nullptr;
+    if (is_q) {
+        dst = q_out + (t * H + head) * D;
+    } else {
+        const int slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
+        if (slot < 0) return;
+        dst = k_cache + ((int64_t)slot * G + (head - H)) * D;
+        raw = v_cache + ((int64_t)slot * G + (head - H)) * D;
+    }
+    const int e0 = 2 * lane;
+    const bool live = e0 < D;
+    float x0 = 0.f, x1 = 0.f;
+    if (live) {
+        SsPair<T>::load(src + e0, x0, x1);
+        if (raw != nullptr) SsPair<T>::copy(raw + e0, src + e0);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(x0 * x0 + x1 * x1) / (float)D + eps);
+    float y0 = 0.f, y1 = 0.f;
+    if (live) {
+        y0 = x0 * rstd * w[e0];
+        y1 = x1 * rstd * w[e0 + 1];
+    }
+    const int half = rot_dims >> 1;
+    const bool turns = e0 < rot_dims, low = e0 < half;
+    const int partner = turns ? (low ? lane + (half >> 1) : lane - (half >> 1)) : lane;
+    const float p0 = __shfl(y0, partner), p1 = __shfl(y1, partner);
+    if (turns) {
+        const int i = low ? e0 : e0 - half;
+        const float pos = (float)positions[t];
+        float s0, c0, s1, c1;
+        sincosf(pos * freq[i], &s0, &c0);
+        sincosf(pos * freq[i + 1], &s1, &c1);
+        if (low) {
+            y0 = y0 * c0 - p0 * s0;
+            y1 = y1 * c1 - p1 * s1;
+        } else {
+            y0 = y0 * c0 + p0 * s0;
+            y1 = y1 * c1 + p1 * s1;
+        }
+    }
+    if (live) SsPair<T>::store(dst + e0, y0, y1);
+}
+
 }  // namespace nv
 
 extern "C" int nv_stream_boundary_scaled(void* resid, const void* add1, int64_t add1_stride, const void* add2,
@@ -179,12 +328,17 @@ extern "C" int nv_poly_norm(const void* x, int64_t x_stride, const float* coef, 
     NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_poly_norm: bad dtype");
     NV_REQUIRE(rows < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_poly_norm: launch too large");
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == NV_DTYPE_BF16)
-        hipLaunchKernelGGL(poly_norm_kernel<__bf16>, dim3((unsigned)rows), dim3(kSsThreads), 0, s, (const __bf16*)x, x_stride,
-                           coef, eps, (__bf16*)y, cols);
-    else
-        hipLaunchKernelGGL(poly_norm_kernel<float>, dim3((unsigned)rows), dim3(kSsThreads), 0, s, (const float*)x, x_stride,
-                           coef, eps, (float*)y, cols);
+    const int n = dtype == NV_DTYPE_BF16 ? 8 : 4;              // elements in a 16-byte piece
+    const bool vec = cols % n == 0 && x_stride % n == 0 && ((uintptr_t)x | (uintptr_t)y) % 16 == 0;
+#define NV_POLY(T, V)                                                                                                \
+    hipLaunchKernelGGL((poly_norm_kernel<T, V>), dim3((unsigned)rows), dim3(kSsThreads), 0, s, (const T*)x, x_stride, coef, \
+                       eps, (T*)y, cols)
+    if (dtype == NV_DTYPE_BF16) {
+        if (vec) NV_POLY(__bf16, true); else NV_POLY(__bf16, false);
+    } else {
+        if (vec) NV_POLY(float, true); else NV_POLY(float, false);
+    }
+#undef NV_POLY
     return check_launch("nv_poly_norm");
 }
 
@@ -203,13 +357,19 @@ extern "C" int nv_head_norm_rope_store(const void* q, const void* k, int64_t q_s
     const int64_t items = T * (H + G), grid = (items + 3) / 4;
     NV_REQUIRE(grid < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_head_norm_rope_store: launch too large");
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == NV_DTYPE_BF16)
-        hipLaunchKernelGGL(head_norm_rope_store_kernel<__bf16>, dim3((unsigned)grid), dim3(256), 0, s, (const __bf16*)q,
-                           (const __bf16*)k, q_stride, k_stride, q_norm, k_norm, eps, freq, rot_dims, positions, slot_mapping,
-                           (__bf16*)q_out, (__bf16*)k_cache, (__bf16*)v_cache, items, H, G, D);
-    else
-        hipLaunchKernelGGL(head_norm_rope_store_kernel<float>, dim3((unsigned)grid), dim3(256), 0, s, (const float*)q,
-                           (const float*)k, q_stride, k_stride, q_norm, k_norm, eps, freq, rot_dims, positions, slot_mapping,
-                           (float*)q_out, (float*)k_cache, (float*)v_cache, items, H, G, D);
+    // two dimensions per lane: even sizes that fit one wave, rotary halves of an even number of dimensions, and rows that
+    // start on the pair's alignment
+    const uintptr_t align = dtype == NV_DTYPE_BF16 ? 4 : 8;
+    const bool pairs = D <= 128 && D % 2 == 0 && rot_dims % 4 == 0 && q_stride % 2 == 0 && k_stride % 2 == 0 &&
+                       ((uintptr_t)q | (uintptr_t)k | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache) % align == 0;
+#define NV_HNR(KERNEL, T)                                                                                                  \
+    hipLaunchKernelGGL(KERNEL<T>, dim3((unsigned)grid), dim3(256), 0, s, (const T*)q, (const T*)k, q_stride, k_stride, q_norm, \
+                       k_norm, eps, freq, rot_dims, positions, slot_mapping, (T*)q_out, (T*)k_cache, (T*)v_cache, items, H, G, D)
+    if (dtype == NV_DTYPE_BF16) {
+        if (pairs) NV_HNR(head_norm_rope_store_pairs_kernel, __bf16); else NV_HNR(head_norm_rope_store_kernel, __bf16);
+    } else {
+        if (pairs) NV_HNR(head_norm_rope_store_pairs_kernel, float); else NV_HNR(head_norm_rope_store_kernel, float);
+    }
+#undef NV_HNR
     return check_launch("nv_head_norm_rope_store");
 }
