@@ -237,57 +237,54 @@ __global__ __launch_bounds__(256) void head_norm_rope_store_pairs_kernel(
     const T* __restrict__ q, const T* __restrict__ k, int64_t q_stride, int64_t k_stride, const float* __restrict__ q_norm,
     const float* __restrict__ k_norm, float eps, const float* __restrict__ freq, int rot_dims,
     const int64_t* __restrict__ positions, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
-    T* __restrict__ k_cache, T* __restrict__ v_cache, int64_t items, int H, int G, int D) {
-    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= items) return;                         // (whole waves leave together)
-    const int lane = threadIdx.x & 63;
-    const int64_t t = item / (H + G);
-    const int head = (int)(item - t * (H + G));
-    const bool is_q = head < H;
-    const T* src = is_q ? q + t * q_stride + (int64_t)head * D : k + t * k_stride + (int64_t)(head - H) * D;
-    const float* w = is_q ? q_norm : k_norm;
-    T* dst;
-    T* raw = nullptr;
-    if (is_q) {
-        dst = q_out + (t * H + head) * D;
-    } else {
-        const int slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
-        if (slot < 0) return;
-        dst = k_cache + ((int64_t)slot * G + (head - H)) * D;
-        raw = v_cache + ((int64_t)slot * G + (head - H)) * D;
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int D) {
+    // A workgroup per token: the token's cosines and sines are computed once (full-precision argument reduction is the
+    // expensive part of this kernel) and shared by the waves, which take the token's heads in turn.
+    __shared__ float cs[2][64];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int half = rot_dims >> 1;
+    if ((int)threadIdx.x < half) {
+        const float ang = (float)positions[t] * freq[threadIdx.x];
+        sincosf(ang, &cs[1][threadIdx.x], &cs[0][threadIdx.x]);
     }
+    __syncthreads();
+    const int slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
     const int e0 = 2 * lane;
     const bool live = e0 < D;
-    float x0 = 0.f, x1 = 0.f;
-    if (live) {
-        SsPair<T>::load(src + e0, x0, x1);
-        if (raw != nullptr) SsPair<T>::copy(raw + e0, src + e0);
-    }
-    const float rstd = 1.0f / sqrtf(wave_sum(x0 * x0 + x1 * x1) / (float)D + eps);
-    float y0 = 0.f, y1 = 0.f;
-    if (live) {
-        y0 = x0 * rstd * w[e0];
-        y1 = x1 * rstd * w[e0 + 1];
-    }
-    const int half = rot_dims >> 1;
     const bool turns = e0 < rot_dims, low = e0 < half;
     const int partner = turns ? (low ? lane + (half >> 1) : lane - (half >> 1)) : lane;
-    const float p0 = __shfl(y0, partner), p1 = __shfl(y1, partner);
-    if (turns) {
-        const int i = low ? e0 : e0 - half;
-        const float pos = (float)positions[t];
-        float s0, c0, s1, c1;
-        sincosf(pos * freq[i], &s0, &c0);
-        sincosf(pos * freq[i + 1], &s1, &c1);
-        if (low) {
-            y0 = y0 * c0 - p0 * s0;
-            y1 = y1 * c1 - p1 * s1;
-        } else {
-            y0 = y0 * c0 + p0 * s0;
-            y1 = y1 * c1 + p1 * s1;
+    const int pair = turns ? (low ? e0 : e0 - half) : 0;
+    for (int head = wave; head < H + G; head += 4) {
+        const bool is_q = head < H;
+        if (!is_q && slot < 0) break;                  // (the wave's later heads are key heads too)
+        const T* src = is_q ? q + t * q_stride + (int64_t)head * D : k + t * k_stride + (int64_t)(head - H) * D;
+        const float* w = is_q ? q_norm : k_norm;
+        T* dst = is_q ? q_out + (t * H + head) * D : k_cache + ((int64_t)slot * G + (head - H)) * D;
+        float x0 = 0.f, x1 = 0.f;
+        if (live) {
+            SsPair<T>::load(src + e0, x0, x1);
+            if (!is_q) SsPair<T>::copy(v_cache + ((int64_t)slot * G + (head - H)) * D + e0, src + e0);
         }
+        const float rstd = 1.0f / sqrtf(wave_sum(x0 * x0 + x1 * x1) / (float)D + eps);
+        float y0 = 0.f, y1 = 0.f;
+        if (live) {
+            y0 = x0 * rstd * w[e0];
+            y1 = x1 * rstd * w[e0 + 1];
+        }
+        const float p0 = __shfl(y0, partner), p1 = __shfl(y1, partner);
+        if (turns) {
+            const float c0 = cs[0][pair], s0 = cs[1][pair], c1 = cs[0][pair + 1], s1 = cs[1][pair + 1];
+            if (low) {
+                y0 = y0 * c0 - p0 * s0;
+                y1 = y1 * c1 - p1 * s1;
+            } else {
+                y0 = y0 * c0 + p0 * s0;
+                y1 = y1 * c1 + p1 * s1;
+            }
+        }
+        if (live) SsPair<T>::store(dst + e0, y0, y1);
     }
-    if (live) SsPair<T>::store(dst + e0, y0, y1);
 }
 
 }  // namespace nv
@@ -362,14 +359,21 @@ extern "C" int nv_head_norm_rope_store(const void* q, const void* k, int64_t q_s
     const uintptr_t align = dtype == NV_DTYPE_BF16 ? 4 : 8;
     const bool pairs = D <= 128 && D % 2 == 0 && rot_dims % 4 == 0 && q_stride % 2 == 0 && k_stride % 2 == 0 &&
                        ((uintptr_t)q | (uintptr_t)k | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache) % align == 0;
-#define NV_HNR(KERNEL, T)                                                                                                  \
-    hipLaunchKernelGGL(KERNEL<T>, dim3((unsigned)grid), dim3(256), 0, s, (const T*)q, (const T*)k, q_stride, k_stride, q_norm, \
-                       k_norm, eps, freq, rot_dims, positions, slot_mapping, (T*)q_out, (T*)k_cache, (T*)v_cache, items, H, G, D)
+#define NV_HNR(T)                                                                                                          \
+    hipLaunchKernelGGL(head_norm_rope_store_kernel<T>, dim3((unsigned)grid), dim3(256), 0, s, (const T*)q, (const T*)k, q_stride, \
+                       k_stride, q_norm, k_norm, eps, freq, rot_dims, positions, slot_mapping, (T*)q_out, (T*)k_cache,             \
+                       (T*)v_cache, items, H, G, D)
+#define NV_HNR_PAIRS(T)                                                                                                    \
+    hipLaunchKernelGGL(head_norm_rope_store_pairs_kernel<T>, dim3((unsigned)T_rows), dim3(256), 0, s, (const T*)q, (const T*)k, \
+                       q_stride, k_stride, q_norm, k_norm, eps, freq, rot_dims, positions, slot_mapping, (T*)q_out,             \
+                       (T*)k_cache, (T*)v_cache, H, G, D)
+    const int64_t T_rows = T;
     if (dtype == NV_DTYPE_BF16) {
-        if (pairs) NV_HNR(head_norm_rope_store_pairs_kernel, __bf16); else NV_HNR(head_norm_rope_store_kernel, __bf16);
+        if (pairs) NV_HNR_PAIRS(__bf16); else NV_HNR(__bf16);
     } else {
-        if (pairs) NV_HNR(head_norm_rope_store_pairs_kernel, float); else NV_HNR(head_norm_rope_store_kernel, float);
+        if (pairs) NV_HNR_PAIRS(float); else NV_HNR(float);
     }
 #undef NV_HNR
+#undef NV_HNR_PAIRS
     return check_launch("nv_head_norm_rope_store");
 }
