@@ -216,3 +216,19 @@ def test_head_sizes_of_the_tile_kernels_through_the_engine(dtype):
     p = {"a": tokens(333, 22), "b": tokens(70, 23), "c": tokens(150, 24)}
     eng = make_engine(cfg, ck, "cuda", dtype, block_size=16, num_blocks=64)
     check(eng, cfg, ck, p, {"a": [130, 1, 67, 64, 1, 70], "b": [1], "c": [65, 2, 83]}, dtype, order={"b": 1, "c": 2})
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_the_largest_head_sizes_through_the_engine(dtype):
+    """Memories of up to 256 x 256 channels (64 key rows per lane, the 1024-thread instantiation, fewer tokens per LDS
+    tile) and attention heads of 160 and 256 dimensions (the one-dimension-per-lane norm kernel, the wide attention
+    tiles), eleven taps (beyond the register window)."""
+    cfg = config([mlstm_layer(heads=1, dim=200, vdim=160, mlp=None), hgrn2_layer(heads=1, dim=256, vdim=256, mlp=dense(96)),
+                  attention_layer(heads=2, kv_heads=1, dim=160, conv=11, rot_dims=64, mlp=None),
+                  attention_layer(heads=2, kv_heads=2, dim=256, conv=2, rot_dims=256, scaling=None, mlp=moe(experts=4, top=2, ff=40, groups=2, keep=2, shared=33))],
+                 width=48)
+    ck = random_checkpoint(cfg, seed=41)
+    p = {"a": tokens(150, 42), "b": tokens(40, 43)}
+    eng = make_engine(cfg, ck, "cuda", dtype, block_size=16, num_blocks=24)
+    check(eng, cfg, ck, p, {"a": [70, 1, 2, 66, 1], "b": [1]}, dtype, order={"b": 1})
