@@ -110,10 +110,11 @@ def test_random_configuration(seed, backend):
         limit = 3 * torch.clamp(noise, min=noise.median().item()) + 1e-3
         over = (err > limit).nonzero().flatten().tolist()
         if len(over) > max(1, err.numel() // 10):
-            # one event (a router's close call, a normaliser that crosses zero) and its fading trail through the states
-            # of one sequence is rounding too: the first excess is then the largest and all lie in that sequence
+            # one event (a router's close call, a normaliser that crosses zero) and its fading trail through the states of
+            # its sequence is rounding too: the positions behind the largest excess, in the same sequence, do not count
             ends = torch.tensor([len(p[i]) for i in p]).cumsum(0).tolist()
-            owner = lambda at: next(j for j, e in enumerate(ends) if at < e)
-            assert len({owner(at) for at in over}) == 1 and err[over[0]] == err[over].max() and len(over) <= err.numel() // 5, \
-                (seed, (err / limit).topk(5).values.tolist())
+            worst = int((err / limit).argmax())
+            end = next(e for e in ends if worst < e)
+            over = [at for at in over if not worst < at < end]
+        assert len(over) <= max(1, err.numel() // 10), (seed, (err / limit).topk(5).values.tolist())
         assert err.median().item() <= 2 * noise.median().item() + 1e-3, (seed, err.median().item(), noise.median().item())
