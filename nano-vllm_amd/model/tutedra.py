@@ -282,8 +282,11 @@ class TutedraAttention(nn.Module, _FusedInputs):
     def forward(self, h, positions, caches):
         m = self.m
         nq = m.heads * m.dim
-        qk = torch.cat(self._project(h, self._inputs), dim=1) if getattr(self, "_fused_w", None) is None \
-            or self._fused_w.device != h.device or self._fused_w.dtype != h.dtype else F.linear(h, self._fused_w)
+        w = getattr(self, "_fused_w", None)
+        if w is not None and w.device == h.device and w.dtype == h.dtype:
+            qk = F.linear(h, w)                                    # [q | k] rows of one product
+        else:
+            qk = torch.cat(self._project(h, self._inputs), dim=1)
         if self.conv is not None:
             qk = self.conv(qk, caches[1]["conv"])
         o = self.attn(qk[:, :nq].unflatten(1, (m.heads, m.dim)), qk[:, nq:].unflatten(1, (m.kv_heads, m.dim)), positions,
@@ -320,7 +323,7 @@ class TutedraMoE(nn.Module):
             self.shared_act = L.ReluSquared()
 
     def forward(self, h, h32):
-        ids, weights = self.router(F.linear(h32, self.router_weight))
+        ids, weights = self.router(F.linear(h32 if h32 is not None else h, self.router_weight))
         out = dict(parts=self.experts(h, ids, weights, self.up, self.down))
         if self.c.shared_ff:
             z = self.shared_in(h)
@@ -408,19 +411,27 @@ class TutedraForCausalLM(nn.Module):
             for i, layer in enumerate(self.layers):
                 p = f"l{i}."
                 layer.mix.place(p + "mix.", take)
+                dev = layer.norm1.weight.device
                 for name in ("ls1", "ls2"):
-                    if getattr(layer, name) is not None:
-                        if p + name in tensors:
-                            getattr(layer, name).copy_(take(p + name).reshape(W))
-                        else:
-                            setattr(layer, name, None)
+                    if name == "ls2" and layer.mlp is None:
+                        continue
+                    if p + name in tensors:
+                        if getattr(layer, name) is None:
+                            setattr(layer, name, nn.Parameter(torch.ones(W, dtype=torch.float32, device=dev)))
+                        getattr(layer, name).copy_(take(p + name).reshape(W))
+                    else:
+                        setattr(layer, name, None)
                 if p + "shift" in tensors:
+                    if layer.shift is None:
+                        layer.shift = self._L.TokenShiftMix(1, W, device=dev)
                     layer.shift.mu[0].copy_(take(p + "shift").reshape(W))
                 else:
                     layer.shift = None
                 if isinstance(layer.mlp, TutedraMoE):
                     mlp, c = layer.mlp, layer.mlp.c
                     if p + "mlp.correction" in tensors:
+                        if mlp.router.correction is None:
+                            mlp.router.correction = nn.Parameter(torch.zeros(c.experts, dtype=torch.float32, device=dev))
                         mlp.router.correction.copy_(take(p + "mlp.correction").reshape(c.experts))
                     else:
                         mlp.router.correction = None
@@ -503,8 +514,9 @@ class TutedraForCausalLM(nn.Module):
                     x, y, logits_rows = x[logits_rows], y[logits_rows], None
                 _, h = boundary(x, add=y, col_scale=layer.ls1, norm=nxt, eps=eps, out_dtype=dt)
             else:
+                # a router reads the norm in float32 (in a float32 model that is h itself)
                 h32, h = boundary(x, add=y, col_scale=layer.ls1, norm=layer.norm2.applied, eps=eps, out_dtype=dt,
-                                  want_f32=isinstance(layer.mlp, TutedraMoE))
+                                  want_f32=isinstance(layer.mlp, TutedraMoE) and dt != torch.float32)
                 if cut:
                     h32 = h32[logits_rows] if h32 is not None else None
                     x, h, logits_rows = x[logits_rows], h[logits_rows], None

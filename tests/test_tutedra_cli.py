@@ -113,3 +113,19 @@ def test_generate_program_matches_the_oracle_greedy(tmp_path):
     for _ in range(6):
         seq.append(int(oracle_logits(CFG, ck, seq)[-1].argmax()))
     assert out["token_ids"] == seq[len(prompt):]
+
+
+def test_a_model_can_be_loaded_again_with_other_optional_tensors():
+    cfg = config([mlstm_layer(mlp=moe())])
+    from tutedra_util import make_engine
+    full, bare = random_checkpoint(cfg, 5), random_checkpoint(cfg, 5, scales=False, shift=False, correction=False)
+    eng = make_engine(cfg, bare, "cpu")
+    layer = eng.runner.model.layers[0]
+    assert layer.ls1 is None and layer.ls2 is None and layer.shift is None and layer.mlp.router.correction is None
+    toks = list(range(2, 21))
+    got = eng.replay_step([("a", toks, list(range(len(toks))))], ["a"])
+    assert rel_err(got, oracle_logits(cfg, bare, toks)) < 5e-5
+    eng.runner.model.load_tensors(full)
+    assert layer.ls1 is not None and layer.shift is not None and layer.mlp.router.correction is not None
+    got = eng.replay_step([("b", toks, list(range(len(toks))))], ["b"])
+    assert rel_err(got, oracle_logits(cfg, full, toks)) < 5e-5
